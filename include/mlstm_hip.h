@@ -64,6 +64,20 @@ int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f,
                      size_t workspace_bytes, void* stream);
 
 /*
+ * mlstm_forward_ex for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and results as
+ * mlstm_forward_ex without the workspace: the scratch is a static device array of MLSTM_NOALLOC_MAX_WORKSPACE bytes
+ * inside the library (each GPU the library runs on holds one until the process ends), and the call performs no
+ * hipMalloc / hipFree, stream-ordered or otherwise.  Shapes whose mlstm_workspace_bytes(MLSTM_OP_FORWARD, ...) exceeds
+ * that size are rejected with MLSTM_EWORKSPACE.  All calls on one GPU share the one array: two calls that overlap in
+ * time on the same GPU (different streams or threads) race; calls on one stream are ordered and safe.
+ * (With mlstm_timing_enable on, events are created around the launches; leave it off in such callers.)
+ */
+#define MLSTM_NOALLOC_MAX_WORKSPACE (8u << 20)
+int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m,
+                             float* b, int B, int NH, int S, int D, int dtype, int gate_dtype, void* stream);
+
+/*
  * General backward: what Triton_mLSTM.backward launches,
  *   mlstm_matmul_kernel_backward_db / _backward / _df           (mlstm_matmul.py:133-333, :384-405).
  * h, m, b are the forward's outputs (h in `dtype`, m and b fp32); any of them may be NULL, in which case all

@@ -9,6 +9,7 @@ LIB_PATH = os.path.join(_HERE, "libmlstm_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 OP_FORWARD, OP_BACKWARD, OP_SCAN_FORWARD, OP_FORWARD_GATED, OP_BACKWARD_GATED = 0, 1, 2, 3, 4
+NOALLOC_MAX_WORKSPACE = 8 << 20   # MLSTM_NOALLOC_MAX_WORKSPACE
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dtype)",
            -2: "unsupported shape (head dimension / sequence length)",
@@ -36,6 +37,8 @@ def lib():
         L.mlstm_backward.argtypes = [vp] * 13 + [ctypes.c_uint]
         L.mlstm_forward_ex.restype = ci
         L.mlstm_forward_ex.argtypes = [vp] * 8 + [ci] * 6 + [vp, sz, vp]
+        L.mlstm_forward_noalloc_ex.restype = ci
+        L.mlstm_forward_noalloc_ex.argtypes = [vp] * 8 + [ci] * 6 + [vp]
         L.mlstm_backward_ex.restype = ci
         L.mlstm_backward_ex.argtypes = [vp] * 14 + [ci] * 6 + [vp, sz, vp]
         L.mlstm_saved_state_bytes.restype = sz
@@ -67,7 +70,7 @@ def lib():
 
 
 def exported_symbols():
-    return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
+    return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",

@@ -112,6 +112,32 @@ struct Scratch {
     ~Scratch() { if (owned && p) (void)hipFreeAsync(p, st); }
 };
 
+// Scratch of mlstm_forward_noalloc_ex: the forward's workspace as a file-scope device array, for callers that cannot
+// allocate.  Every GPU the library runs on holds its own copy at its own address until the process ends; in host code
+// the array's name is only a handle for hipGetSymbolAddress, never a device address, so the address is looked up once
+// per device (with that device current) and everything after that -- kernel arguments included -- uses the pointer.
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)MLSTM_NOALLOC_MAX_WORKSPACE;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+constexpr int NOALLOC_MAX_DEVICES = 64;
+void* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+std::mutex g_scratch_mu;
+int scratch_of_current_device(char** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return MLSTM_EINVAL;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return (int)hipErrorInvalidSymbol;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = static_cast<char*>(g_scratch_ptr[dev]);
+    return 0;
+}
+
 // the first Sizes::fwd() bytes of every workspace
 struct FwdWs {
     double* G2; float *alpha2, *beta2, *ek2, *amax2, *mw, *bw;
@@ -268,6 +294,21 @@ int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f,
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
+}
+
+int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
+                             int B, int NH, int S, int D, int dtype, int gate_dtype, void* stream) {
+    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) || !good_dtype(gate_dtype))
+        return MLSTM_EINVAL;
+    if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    if (z.fwd() > NOALLOC_SCRATCH_BYTES) return MLSTM_EWORKSPACE;   // the shape needs more scratch than the array holds
+    char* ws = nullptr;
+    if (int rc = scratch_of_current_device(&ws)) return rc;
+    // Nothing in the workspace has to start at zero: the gate pre-pass writes every element the tile kernels read,
+    // padding included, and the states are written before they are read; what the previous call left is overwritten.
+    return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, ws, st);
 }
 
 size_t mlstm_saved_state_bytes(int B, int NH, int S, int D, int dtype) {
