@@ -22,6 +22,19 @@ extern "C" {
 #define MLSTM_F16 1
 #define MLSTM_BF16 2
 
+/*
+ * Split mode, or-ed into the `dtype` argument of the *_ex entry points (16-bit types; no effect on MLSTM_F32).
+ * The 16-bit kernels round the weights C~ (and their backward counterparts) to the element type before the second
+ * product of a tile, as every tensor-core implementation does; an output element is a sum of terms that can be far
+ * larger than the element itself, so that rounding shows as an absolute error of about 2^-9 (bf16) of the terms'
+ * size.  With MLSTM_PRECISE every such operand enters its product as two terms, hi + lo, each in the element type
+ * (two MFMAs per fragment), and the forward hands the low-order part of h to the backward (the `saved` buffer of
+ * mlstm_forward_save_ex, or a recomputation), which makes the results agree with an fp32 evaluation of the
+ * reference's formulas (mlstm_matmul.py:104-118, :336-365) to rtol 2e-2 / atol 2e-3 element by element.  Price:
+ * the generic kernels without chunking, and half as many MFMAs again.
+ */
+#define MLSTM_PRECISE 0x100
+
 /* argument errors */
 #define MLSTM_EINVAL (-1)      /* null pointer, non-positive size, unknown dtype */
 #define MLSTM_ESHAPE (-2)      /* head dimension / sequence length not supported by this build */

@@ -229,3 +229,150 @@ def make_inputs(B, NH, S, D, dtype=torch.float32, seed=0, f_mean=0.0, i_mean=0.0
     if with_o:
         out.append(torch.randn((B, NH, S, D), generator=g))
     return [x.to(dtype) for x in out]
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# 16-bit weights.  The reference's Triton kernels are fp32 (mlstm_matmul.py:19, :35 "TODO FP 16"); its CUDA kernels
+# feed the second product of a tile with the weights rounded to half (cuda-src/mlstm_forward.cu:143-160,
+# cutlass-src-ampere/mlstm_forward.cu:308-313), as every tensor-core pipeline does.  The two functions below restate
+# that algorithm on the CPU and predict the size of its rounding noise, so that a 16-bit kernel can be held to the
+# algorithm it implements, and the distance of that algorithm from the fp32 formulas can be measured rather than
+# absorbed into a tolerance.
+# ---------------------------------------------------------------------------------------------------------------
+def _round_to(x, dtype, terms):
+    """x rounded to ``dtype`` as a sum of ``terms`` values of that type (1: plain rounding, 2: hi + lo)."""
+    hi = x.to(dtype).to(x.dtype)
+    if terms == 1:
+        return hi
+    return hi + (x - hi).to(dtype).to(x.dtype)
+
+
+def mlstm_rounded_weights_dense(dh, q, k, v, f, i, dtype, terms=1):
+    """Forward and backward (mlstm_matmul.py:104-118, :336-365) with the operands a 16-bit kernel rounds to the
+    element type before a tile's second product: C~ (forward, ``P``), dC~ D' (``G``, dQ and dK), C~ / n (``W``, dV),
+    and the forward output h where the backward uses it for dn = -(dh . h) / n.  Everything else in float64.
+    ``terms=2`` is the split mode (each operand as hi + lo).  Returns (h, dq, dk, dv, df, di), unrounded float64."""
+    dh, q, k, v, f, i = (_up(x, torch.float64) for x in (dh, q, k, v, f, i))
+    B, NH, S, D = q.shape
+    outs = [torch.empty_like(q) for _ in range(4)] + [torch.empty_like(f), torch.empty_like(f)]
+    sc = 1.0 / math.sqrt(D)
+    rnd = lambda x: _round_to(x, dtype, terms)
+    for bi in range(B):
+        for hi_ in range(NH):
+            Q, K, V, dH = q[bi, hi_], k[bi, hi_], v[bi, hi_], dh[bi, hi_]
+            d, m = _decay_matrix(f[bi, hi_], i[bi, hi_])
+            dp = torch.exp(d - m[:, None])
+            ct = (Q @ K.T) * sc * dp
+            b = ct.sum(-1)
+            n = torch.maximum(b.abs(), torch.exp(-m)) + EPS
+            h = (rnd(ct) @ V) / n[:, None]
+            dn = -(dH * rnd(h)).sum(-1) / n
+            db = torch.sign(b) * dn * (b.abs() > torch.exp(-m)).to(torch.float64)
+            dct = (dH @ V.T) / n[:, None] + db[:, None]
+            G = rnd(dct * dp * sc)
+            dD = ct * dct
+            cs = torch.cumsum(dD.sum(-2) - dD.sum(-1), -1)
+            g = torch.roll(cs, 1, -1)
+            g[0] = 0.0
+            for o_, val in zip(outs, (h, G @ K, G.T @ Q, rnd(ct / n[:, None]).T @ dH, torch.sigmoid(-f[bi, hi_]) * g, dD.sum(-2))):
+                o_[bi, hi_] = val
+    return tuple(outs)
+
+
+def rounding_unit_std(dtype):
+    """Standard deviation of the relative error of round-to-nearest into ``dtype``, taken at its largest (values just
+    above a power of two): ulp / sqrt(12) with ulp = 2^-7 (bfloat16: 8 significant bits) or 2^-10 (float16: 11)."""
+    return {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[dtype] / math.sqrt(12.0)
+
+
+def mlstm_rounding_noise(dh, q, k, v, f, i, dtype, work_dtype=torch.float64, chunk_len=0):
+    """Per-element standard deviation of the error that rounding P, G, W and h to ``dtype`` (see
+    mlstm_rounded_weights_dense) leaves in h, dq, dk, dv, df, di, under the usual model of independent rounding errors:
+    an output that is sum_j w_j x_j with w rounded has variance u^2 sum_j (w_j x_j)^2, u = rounding_unit_std.  The
+    rounding of h enters through db_i = +-(dh_i . h_i) / n_i, which is common to a whole row of dC~ (and of dD, whose
+    sums are di and, cumulatively, df).
+
+    ``chunk_len`` = L > 0 models an evaluation in chunks of L positions, where a row meets the keys before its chunk
+    through the matrix state of the scan form (mlstm_scan.py:16-26) at the end of the previous chunk, C~ = sum_j w_j k_j
+    v_j^T / sqrt(D), and a key meets the queries behind its chunk through the mirror-image state E = sum_i rho_i / n_i
+    q_i dh_i^T / sqrt(D), both stored in ``dtype``: every output gains the rounding of the state it is contracted
+    with, and the row and column sums of dD of those far pairs, now q_i . dQ_i and k_j . dK_j, gain a per-position
+    error that the running sum of df accumulates between the chunk boundaries, where it is pinned to sum <C~, E>
+    (a bridge: what a chunk's own sum misses of the next pinned value is spread evenly over the chunk).
+
+    Returns a tuple of tensors shaped like the outputs, in ``work_dtype`` (float32 halves the memory of the S x S
+    intermediates of very long sequences)."""
+    dh, q, k, v, f, i = (_up(x, work_dtype) for x in (dh, q, k, v, f, i))
+    B, NH, S, D = q.shape
+    u2 = rounding_unit_std(dtype) ** 2
+    outs = [torch.empty_like(q) for _ in range(4)] + [torch.empty_like(f), torch.empty_like(f)]
+    sc = 1.0 / math.sqrt(D)
+    L = int(chunk_len)
+    ncs = (S - 1) // L if L > 0 else 0          # complete chunks with something behind them
+    for bi in range(B):
+        for hi_ in range(NH):
+            Q, K, V, dH = q[bi, hi_], k[bi, hi_], v[bi, hi_], dh[bi, hi_]
+            d, m = _decay_matrix(f[bi, hi_], i[bi, hi_])
+            dp = torch.exp(d - m[:, None])
+            ct = (Q @ K.T) * sc * dp
+            b = ct.sum(-1)
+            n = torch.maximum(b.abs(), torch.exp(-m)) + EPS
+            h = (ct @ V) / n[:, None]
+            active = (b.abs() > torch.exp(-m)).to(work_dtype)
+            dn = -(dH * h).sum(-1) / n
+            db = torch.sign(b) * dn * active
+            dct = (dH @ V.T) / n[:, None] + db[:, None]
+            G = dct * dp * sc
+            W = ct / n[:, None]
+            var_h = u2 * ((ct ** 2) @ (V ** 2)) / (n * n)[:, None]
+            var_dq = u2 * ((G ** 2) @ (K ** 2))
+            var_dk = u2 * ((G ** 2).T @ (Q ** 2))
+            var_dv = u2 * ((W ** 2).T @ (dH ** 2))
+            var_x = torch.zeros(S, dtype=work_dtype)     # per-position error of (column sum - row sum) of dD, far pairs
+            if ncs > 0:
+                pos = torch.arange(S)
+                cidx = torch.clamp(pos // L, max=ncs)
+                far = (cidx[:, None] > cidx[None, :]).to(work_dtype)          # [row s, key j]: j in an earlier chunk
+                T = ((dH / n[:, None]) ** 2) @ (V ** 2).T                     # sum_v (dh_sv v_jv / n_s)^2
+                pair = u2 * far * ct ** 2 * T                                 # far pairs seen through rounded chunk sums
+                var_x += pair.sum(-1) + pair.sum(-2)
+                for c in range(ncs):
+                    e = (c + 1) * L - 1
+                    rows = slice(e + 1, min(e + 1 + L, S)) if c + 1 < ncs else slice(e + 1, S)   # the rows that read C~_c
+                    keys = slice(c * L, e + 1)                                                      # the keys that read E_c
+                    Cst = (K * (sc * dp[e])[:, None]).T @ V                                         # [key index, value index]
+                    rho = torch.where(pos > e, dp[:, e] / dp[e, e], torch.zeros((), dtype=work_dtype))
+                    Est = (Q * (sc * rho / n)[:, None]).T @ dH
+                    dec2 = ((dp[rows, e] / dp[e, e]) / n[rows]) ** 2
+                    w2 = dp[e, keys] ** 2
+                    var_h[rows] += u2 * ((Q[rows] ** 2) @ (Cst ** 2)) * (dp[rows, e] / dp[e, e] / n[rows])[:, None] ** 2
+                    var_dq[rows] += u2 * ((dH[rows] ** 2) @ (Cst ** 2).T) * dec2[:, None]
+                    var_dv[keys] += u2 * ((K[keys] ** 2) @ (Est ** 2)) * w2[:, None]
+                    var_dk[keys] += u2 * ((V[keys] ** 2) @ (Est ** 2).T) * w2[:, None]
+                    var_x[rows] += u2 * dec2 * (((Q[rows] ** 2) @ (Cst ** 2)) * dH[rows] ** 2).sum(-1)
+                    var_x[keys] += u2 * w2 * (((K[keys] ** 2) @ (Est ** 2)) * V[keys] ** 2).sum(-1)
+            # the h the backward reads carries the noise of the forward's own P as well as its final rounding
+            var_db = ((dH ** 2) * (var_h + u2 * h ** 2)).sum(-1) / (n * n) * active   # [S] variance of db_i
+            var_dq = var_dq + var_db[:, None] * ((dp * sc) @ K) ** 2
+            var_dk = var_dk + ((dp * sc) ** 2).T @ (var_db[:, None] * Q ** 2)
+            var_di = (ct ** 2).T @ var_db + var_x                               # dD_ij moves by ct_ij * (error of db_i)
+            # df_t = sigmoid(-f_t) sum_{s<t} (col_s - row_s): row i of dD contributes c_i(t) = sum_{s<t} ct_is - [i<t] b_i
+            cum = torch.cumsum(ct, -1)
+            cum = torch.cat([torch.zeros((S, 1), dtype=cum.dtype), cum[:, :-1]], -1)      # [i, t] = sum_{s<t} ct_is
+            lower = torch.tril(torch.ones((S, S), dtype=cum.dtype), -1).T                   # [i, t] = 1 if i < t
+            coef = cum - lower * b[:, None]
+            var_run = (coef ** 2).T @ var_db
+            if ncs > 0:   # running sum of the per-position errors inside each chunk, bridged where the chunk's end is pinned
+                for c in range(ncs + 1):
+                    lo, hi = c * L, min((c + 1) * L, S) if c < ncs else S
+                    vx = var_x[lo:hi]
+                    P = torch.cumsum(vx, 0) - vx                                # sum over positions before tau
+                    if c < ncs:
+                        tau = torch.arange(hi - lo, dtype=work_dtype) / float(L)
+                        var_run[lo:hi] += (1 - tau) ** 2 * P + tau ** 2 * (vx.sum() - P)
+                    else:
+                        var_run[lo:hi] += P
+            var_df = torch.sigmoid(-f[bi, hi_]) ** 2 * var_run
+            for o_, val in zip(outs, (var_h, var_dq, var_dk, var_dv, var_df, var_di)):
+                o_[bi, hi_] = val.clamp_min(0).sqrt()
+    return tuple(outs)

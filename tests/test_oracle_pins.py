@@ -211,3 +211,53 @@ def test_check_comparator(capsys):
     assert not O.check(a, a + 1.0, name="Y")
     out = capsys.readouterr().out
     assert "X -- EQUAL" in out and "Percentage non-matching" in out
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# 16-bit weights: the CPU restatement of what a 16-bit kernel computes, and the predicted size of its rounding noise
+# ---------------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rounded_weights_restate_the_same_function(dtype):
+    """With the weights as hi + lo the 16-bit algorithm is the fp64 oracle to a few 2^-16; with plain rounding it stays
+    within the unit roundoff of the weights, relative to the size of an element's terms."""
+    q, k, v, f, i, dh = O.make_inputs(1, 2, 96, 32, dtype, seed=3, f_mean=1.0)
+    exact = [O.mlstm_forward_dense(q, k, v, f, i)[0], *O.mlstm_backward_dense(dh, q, k, v, f, i, zero_first_df=True)]
+    split = O.mlstm_rounded_weights_dense(dh, q, k, v, f, i, dtype, terms=2)
+    plain = O.mlstm_rounded_weights_dense(dh, q, k, v, f, i, dtype, terms=1)
+    u = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
+    for name, e, s2, s1 in zip(["h", "dq", "dk", "dv", "df", "di"], exact, split, plain):
+        scale = float(e.abs().max())
+        assert float((s2 - e).abs().max()) <= 64 * u * u * scale + 1e-12, name
+        assert 0 < float((s1 - e).abs().max()) <= 8 * u * scale or name in ("df", "di"), name
+    assert float(split[4][..., 0].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype,S,D,f_mean", [(torch.bfloat16, 200, 64, 3.0), (torch.float16, 130, 32, 0.0), (torch.bfloat16, 160, 32, -4.0)])
+def test_rounding_noise_model_against_the_emulation(dtype, S, D, f_mean):
+    """The predicted standard deviation must describe the emulated 16-bit algorithm's actual error: rms of error / sigma
+    between 0.5 and 1.1 (the model takes the rounding unit at its largest), and no element beyond 5 sigma."""
+    worst, ratio = {}, {}
+    names = ["h", "dq", "dk", "dv", "df", "di"]
+    for seed in range(3):
+        q, k, v, f, i, dh = O.make_inputs(1, 1, S, D, dtype, seed=seed, f_mean=f_mean, i_mean=2.0 if f_mean < 0 else 0.0)
+        exact = [O.mlstm_forward_dense(q, k, v, f, i)[0], *O.mlstm_backward_dense(dh, q, k, v, f, i, zero_first_df=True)]
+        emu = O.mlstm_rounded_weights_dense(dh, q, k, v, f, i, dtype)
+        sig = O.mlstm_rounding_noise(dh, q, k, v, f, i, dtype)
+        for name, e, g, s in zip(names, exact, emu, sig):
+            err = (g - e).abs()
+            live = s > 1e-12 * float(s.max())
+            worst[name] = max(worst.get(name, 0.0), float((err[live] / s[live]).max()))
+            ratio[name] = ratio.get(name, 0.0) + float(err.pow(2).mean().sqrt() / s.pow(2).mean().sqrt()) / 3
+    for name in names:
+        assert worst[name] < 5.0, (name, worst[name])
+        assert 0.5 < ratio[name] < 1.1, (name, ratio[name])
+
+
+def test_rounding_noise_in_chunks_only_adds():
+    q, k, v, f, i, dh = O.make_inputs(1, 1, 300, 32, torch.bfloat16, seed=1, f_mean=4.0)
+    plain = O.mlstm_rounding_noise(dh, q, k, v, f, i, torch.bfloat16)
+    chunks = O.mlstm_rounding_noise(dh, q, k, v, f, i, torch.bfloat16, chunk_len=128)
+    for a, c in zip(plain, chunks):
+        assert bool((c >= a * (1 - 1e-12)).all())
+    assert float(chunks[0][0, 0, 128:].sum()) > float(plain[0][0, 0, 128:].sum())     # rows behind the first chunk read a state
+    assert torch.equal(chunks[0][0, 0, :128], plain[0][0, 0, :128])                  # the first chunk reads none

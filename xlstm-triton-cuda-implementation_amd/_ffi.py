@@ -8,6 +8,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmlstm_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
+PRECISE = 0x100   # MLSTM_PRECISE, or-ed into the dtype code: split mode of the 16-bit kernels
 OP_FORWARD, OP_BACKWARD, OP_SCAN_FORWARD, OP_FORWARD_GATED, OP_BACKWARD_GATED = 0, 1, 2, 3, 4
 NOALLOC_MAX_WORKSPACE = 8 << 20   # MLSTM_NOALLOC_MAX_WORKSPACE
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
@@ -108,9 +109,9 @@ def timing_read(kernel):
     return ms.value, n.value
 
 
-def dtype_code(dt):
+def dtype_code(dt, precise=False):
     try:
-        return _DTYPES[dt]
+        return _DTYPES[dt] | (PRECISE if precise and dt != torch.float32 else 0)
     except KeyError:
         raise TypeError(f"unsupported dtype {dt}; expected float32, float16 or bfloat16") from None
 

@@ -54,8 +54,9 @@ struct Carver {
 // 16-bit types at D >= 128; a chunk pays D/64 state tiles per row tile and saves the key tiles before the chunk, and the
 // states cost 2 S D^2 flops per head whatever the length.
 int g_chunk_override = 0;   // test aid: > 0 forces this length, < 0 switches chunking off
-int chunk_len_for(int dtype, int D, size_t S) {
-    if (dtype == MLSTM_F32 || !(D == 128 || D == 256) || mlstm::g_force_generic || g_chunk_override < 0) return 0;
+int chunk_len_for(int dtype, int D, size_t S, bool precise = false) {
+    // (split mode runs on the generic kernels, which walk every key tile)
+    if (dtype == MLSTM_F32 || !(D == 128 || D == 256) || mlstm::g_force_generic || g_chunk_override < 0 || precise) return 0;
     if (g_chunk_override > 0) return S > (size_t)g_chunk_override ? g_chunk_override : 0;
     return S >= 1024 ? 512 : 0;   // (below two full chunks the state pass costs more than the skipped key tiles)
 }
@@ -67,22 +68,27 @@ struct Sizes {
     // chunked forward: per-chunk sums (fp32), matrix states (element type), vector states
     size_t n_states(int L) const { return L > 0 && S > (size_t)L ? (S - 1) / L : 0; }
     size_t chunk_states(int dtype) const {
-        const size_t n = n_states(chunk_len_for(dtype, (int)D, S));
+        const size_t n = n_states(chunk_len_for(dtype, (int)D, S, precise));
         return up256(BH * n * D * D * 4) + up256(BH * n * D * D * el) + up256(BH * n * D * 4);
     }
     int dtype_code = MLSTM_F32;
-    size_t states_t() const { return up256(BH * n_states(chunk_len_for(dtype_code, (int)D, S)) * D * D * el); }   // value-major copy for the dQ pass
-    size_t saved_vec() const { return up256(BH * n_states(chunk_len_for(dtype_code, (int)D, S)) * D * 4); }
-    // what the backward reuses of a chunked forward: value-major states, vector states, the gate pre-pass
-    size_t saved() const { return n_states(chunk_len_for(dtype_code, (int)D, S)) ? states_t() + saved_vec() + gates() : 0; }
+    bool precise = false;   // split mode (MLSTM_PRECISE): no chunks, and the low-order part of h travels to the backward
+    int chunk_len() const { return chunk_len_for(dtype_code, (int)D, S, precise); }
+    size_t states_t() const { return up256(BH * n_states(chunk_len()) * D * D * el); }   // value-major copy for the dQ pass
+    size_t saved_vec() const { return up256(BH * n_states(chunk_len()) * D * 4); }
+    size_t h_lo() const { return precise ? up256(BH * S * D * el) : 0; }
+    // what the backward reuses of the forward: in chunks the value-major states, the vector states and the gate
+    // pre-pass; in split mode h - (h rounded to the element type)
+    size_t saved() const { return precise ? h_lo() : (n_states(chunk_len()) ? states_t() + saved_vec() + gates() : 0); }
     size_t fwd() const { return gates() + stats() + chunk_states(dtype_code); }
     size_t fwd_fixed() const { return gates() + stats(); }   // offset of the chunk states inside fwd()
     size_t bwd() const {
         return fwd() + up256(BH * S * D * el)                                      // recomputed h
                + 2 * up256(BH * NG * 64 * 4) + states_t()                          // inv_n, db; transposed chunk states
                + 2 * states_t() + saved_vec() + up256(BH * S * 4)                  // reverse states (both layouts, vector); far row sums
-               + up256(BH * n_states(chunk_len_for(dtype_code, (int)D, S)) * 4)    // dF anchors
-               + up256(BH * S * 4) + up256(BH * NG * S * 4);                       // colsum, rowpart
+               + up256(BH * n_states(chunk_len()) * 4)                             // dF anchors
+               + up256(BH * S * 4) + up256(BH * NG * S * 4)                        // colsum, rowpart
+               + h_lo();                                                           // split mode: low-order part of a recomputed h
     }
     // gated backward: the ungated upstream gradient, and (h, m, b) when the caller does not bring them
     size_t bwd_gated() const { return bwd() + 2 * up256(BH * S * D * el) + stats(); }
@@ -96,6 +102,16 @@ void scan_mark(int id, hipStream_t st, bool begin) {
 }
 
 bool good_dtype(int dt) { return dt == MLSTM_F32 || dt == MLSTM_F16 || dt == MLSTM_BF16; }
+// element type code as the caller passes it: one of the three types, optionally with MLSTM_PRECISE
+bool good_dtype_arg(int dt) { return dt >= 0 && good_dtype(dt & ~MLSTM_PRECISE); }
+// (fp32 operands are exact: the flag is accepted and has no effect there)
+bool precise_of(int dt) { return (dt & MLSTM_PRECISE) != 0 && (dt & ~MLSTM_PRECISE) != MLSTM_F32; }
+Sizes sizes_of(int B, int NH, int S, int D, int dtype_arg) {
+    const int dt = dtype_arg & ~MLSTM_PRECISE;
+    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dt), dt};
+    z.precise = precise_of(dtype_arg);
+    return z;
+}
 bool good_shape(int D, int dtype) { return D == 64 || D == 128 || (D == 256 && dtype != MLSTM_F32); }
 
 // RAII for a stream-ordered scratch allocation when the caller brings no workspace
@@ -151,7 +167,7 @@ struct FwdWs {
         amax2 = c.take<float>(z.BH * z.NG * 2 + 64);   // (+64: the row kernels copy 64 floats from each tile's pair on)
         mw = c.take<float>(z.BH * z.S);
         bw = c.take<float>(z.BH * z.S);
-        L = chunk_len_for(dtype, D, z.S);
+        L = z.chunk_len();
         ncs = z.n_states(L);
         dC = c.take<float>(z.BH * ncs * z.D * z.D);
         Cst = c.take<char>(z.BH * ncs * z.D * z.D * z.el);
@@ -181,7 +197,7 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
                  const Sizes& z, int D, int dtype, int gate_dtype, char* ws, hipStream_t st, float** alpha_out = nullptr,
                  float** beta_out = nullptr, double** g_out = nullptr, float** m_out = nullptr, float** b_out = nullptr,
                  float** ek_out = nullptr, float** amax_out = nullptr, const void* o = nullptr, void* h_gated = nullptr,
-                 void* CstT = nullptr, float* Nst_ext = nullptr, char* gates_ext = nullptr) {
+                 void* CstT = nullptr, float* Nst_ext = nullptr, char* gates_ext = nullptr, void* h_lo = nullptr) {
     FwdWs w(ws, z, dtype, D);
     if (gates_ext) w.gates_at(gates_ext, z);
     double* G2 = w.G2; float *alpha2 = w.alpha2, *beta2 = w.beta2, *ek2 = w.ek2, *amax2 = w.amax2;
@@ -197,6 +213,7 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
     a.X = q; a.Y1 = k; a.Y2 = v; a.out = h; a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.Bsum = b;
     a.ek2 = ek2; a.amax2 = amax2; a.O = o; a.out_gated = h_gated;
     a.BH = (int)z.BH; a.S = (int)z.S; a.NG = (int)z.NG;
+    a.precise = z.precise ? 1 : 0; a.out_lo = h_lo;
     if (ncs > 0) {   // long sequence: the states at the chunk ends first, then every row tile stays inside its chunk
         float* Nst = Nst_ext ? Nst_ext : w.Nst;
         if (int e = chunk_states_impl(k, v, w, true, CstT, Nst, z, D, dtype, st)) return e;
@@ -224,8 +241,8 @@ int mlstm_force_generic_kernels(int on) {
 }
 
 int mlstm_chunk_length_for(int S, int D, int dtype) {
-    if (S <= 0 || D <= 0 || !good_dtype(dtype)) return 0;
-    return chunk_len_for(dtype, D, (size_t)S);
+    if (S <= 0 || D <= 0 || !good_dtype_arg(dtype)) return 0;
+    return chunk_len_for(dtype & ~MLSTM_PRECISE, D, (size_t)S, precise_of(dtype));
 }
 
 int mlstm_set_chunk_length(int length) {
@@ -269,8 +286,8 @@ int mlstm_timing_read(int kernel, double* total_ms, int* launches) {
 }
 
 size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype) {
-    if (B <= 0 || NH <= 0 || S <= 0 || D <= 0 || !good_dtype(dtype)) return 0;
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    if (B <= 0 || NH <= 0 || S <= 0 || D <= 0 || !good_dtype_arg(dtype)) return 0;
+    const Sizes z = sizes_of(B, NH, S, D, dtype);
     switch (op) {
         case MLSTM_OP_FORWARD: return z.fwd();
         case MLSTM_OP_BACKWARD: return z.bwd();
@@ -286,11 +303,13 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype) {
 int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                      int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes,
                      void* stream) {
-    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) || !good_dtype(gate_dtype))
+    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -298,11 +317,13 @@ int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f,
 
 int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                              int B, int NH, int S, int D, int dtype, int gate_dtype, void* stream) {
-    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) || !good_dtype(gate_dtype))
+    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     if (z.fwd() > NOALLOC_SCRATCH_BYTES) return MLSTM_EWORKSPACE;   // the shape needs more scratch than the array holds
     char* ws = nullptr;
     if (int rc = scratch_of_current_device(&ws)) return rc;
@@ -312,23 +333,28 @@ int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const 
 }
 
 size_t mlstm_saved_state_bytes(int B, int NH, int S, int D, int dtype) {
-    if (B <= 0 || NH <= 0 || S <= 0 || D <= 0 || !good_dtype(dtype)) return 0;
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    if (B <= 0 || NH <= 0 || S <= 0 || D <= 0 || !good_dtype_arg(dtype)) return 0;
+    const Sizes z = sizes_of(B, NH, S, D, dtype);
     return z.saved();
 }
 
 int mlstm_forward_save_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                           void* saved, size_t saved_bytes, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace,
                           size_t workspace_bytes, void* stream) {
-    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) || !good_dtype(gate_dtype))
+    if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     if (z.saved() > 0 && (!saved || saved_bytes < z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     char* sv = z.saved() > 0 ? (char*)saved : nullptr;
+    if (z.precise)   // split mode: what the backward reuses is the low-order part of h
+        return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
+                            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, sv);
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
                         nullptr, nullptr, nullptr, sv, sv ? reinterpret_cast<float*>(sv + z.states_t()) : nullptr,
                         sv ? sv + z.states_t() + z.saved_vec() : nullptr);
@@ -337,11 +363,13 @@ int mlstm_forward_save_ex(const void* q, const void* k, const void* v, const voi
 int mlstm_forward_gated_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
                            void* h_gated, float* m, float* b, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace,
                            size_t workspace_bytes, void* stream) {
-    if (!q || !k || !v || !f || !i || !o || !h || !h_gated || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) || !good_dtype(gate_dtype))
+    if (!q || !k || !v || !f || !i || !o || !h || !h_gated || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr,
@@ -376,12 +404,16 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs);
+    char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
     // the column kernel runs in chunks too when it is the 16x16 one (the generic kernels know no chunks)
     // (and only for lengths at which the eight-wave row kernel, which leaves rowinter, is sure to have run)
     const bool col_chunks = w.ncs > 0 && z.NG <= 1024;
 
     float *alpha2, *beta2, *mm, *bb, *ek2, *amax2; double* G2;
-    const bool have_fwd = h && m && b;
+    // Split mode needs h beyond the element type's precision for dh . h: either the forward left the low-order part
+    // (saved), or the forward is run again here
+    const void* h_lo = z.precise ? saved : nullptr;
+    const bool have_fwd = h && m && b && (!z.precise || h_lo);
     if (have_fwd) {
         // gates only: alpha, beta, G (and m again, into the workspace) are cheap to rebuild; so are the chunk states
         G2 = w.G2; alpha2 = w.alpha2; beta2 = w.beta2; ek2 = w.ek2; amax2 = w.amax2; mm = w.mw;
@@ -397,16 +429,18 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
             if (int e = chunk_states_impl(k, v, w, false, CstT, w.Nst, z, D, dtype, st)) return e;   // (the dQ pass wants them value-major only)
     } else {
         int rc = forward_impl(q, k, v, f, i, hbuf, nullptr, nullptr, z, D, dtype, gate_dtype, ws, st, &alpha2, &beta2, &G2, &mm, &bb, &ek2, &amax2,
-                              nullptr, nullptr, CstT);
+                              nullptr, nullptr, CstT, nullptr, nullptr, z.precise ? hlo_buf : nullptr);
         Nst = w.Nst;
         if (rc) return rc;
         h = hbuf;
+        if (z.precise) h_lo = hlo_buf;
     }
     // dQ first: it derives 1/n and db per row from (dh, h, m, b) and leaves them for the column kernel
     RowArgs ra{};
     ra.X = dh; ra.Y1 = v; ra.Y2 = k; ra.out = dq; ra.alpha2 = alpha2; ra.beta2 = beta2; ra.G2 = G2; ra.inv_n = inv_n; ra.db = dbuf;
     ra.ek2 = ek2; ra.amax2 = amax2; ra.Hin = h; ra.Bin = bb; ra.M = mm;
     ra.BH = (int)z.BH; ra.S = (int)z.S; ra.NG = (int)z.NG;
+    ra.precise = z.precise ? 1 : 0; ra.Hin_lo = h_lo;
     if (w.ncs > 0) { ra.chunk_len = w.L; ra.n_states = (int)w.ncs; ra.Cst = CstT; ra.Nst = Nst; ra.Qrow = q; ra.rowinter = rowinter; }
     {
         Timed t(MLSTM_K_ROW_DQ, st);
@@ -425,6 +459,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ca.Q = q; ca.K = k; ca.V = v; ca.dH = dh; ca.dK = dk; ca.dV = dv; ca.colsum = colsum; ca.rowpart = rowpart;
     ca.alpha2 = alpha2; ca.beta2 = beta2; ca.G2 = G2; ca.inv_n = inv_n; ca.db = dbuf;
     ca.BH = (int)z.BH; ca.S = (int)z.S; ca.NG = (int)z.NG;
+    ca.precise = z.precise ? 1 : 0;
     if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ek = Ek; ca.Ev = Ev; ca.gvec = gvec; }
     {
         Timed t(MLSTM_K_COL, st);
@@ -443,12 +478,14 @@ extern "C" {
 int mlstm_backward_ex(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
                       const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, int B, int NH, int S,
                       int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes, void* stream) {
-    if (!dh || !q || !k || !v || !f || !i || !dq || !dk || !dv || !df || !di || B <= 0 || NH <= 0 || S <= 0 || !good_dtype(dtype) ||
+    if (!dh || !q || !k || !v || !f || !i || !dq || !dk || !dv || !df || !di || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) ||
         !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;
     return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -459,11 +496,13 @@ int mlstm_backward_saved_ex(const void* dh, const void* q, const void* k, const 
                             void* di, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes,
                             void* stream) {
     if (!dh || !q || !k || !v || !f || !i || !h || !m || !b || !dq || !dk || !dv || !df || !di || B <= 0 || NH <= 0 || S <= 0 ||
-        !good_dtype(dtype) || !good_dtype(gate_dtype))
+        !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     if (z.saved() > 0 && (!saved || saved_bytes < z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;
@@ -475,11 +514,13 @@ int mlstm_backward_gated_ex(const void* dh_gated, const void* q, const void* k, 
                             const void* h, const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, void* d_o,
                             int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes, void* stream) {
     if (!dh_gated || !q || !k || !v || !f || !i || !o || !dq || !dk || !dv || !df || !di || !d_o || B <= 0 || NH <= 0 || S <= 0 ||
-        !good_dtype(dtype) || !good_dtype(gate_dtype))
+        !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
+    const int dtype_arg = dtype;
+    dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dtype), dtype};
+    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd_gated(), st)) return rc;
     char* ws = (char*)sc.p;

@@ -13,13 +13,14 @@
 // Column sums of dD (= dI) stay in registers for the whole kernel; row sums leave the kernel as one partial per
 // (key tile, query) and are added up by the dF pass, so rows and columns are sums of the very same fp32 products
 // and the cancellation in dF = sigmoid(-f) * cumsum(col - row) stays exact to fp32 round-off.
+#include <mutex>
 #include <type_traits>
 #include "mlstm_common.cuh"
 #include "mlstm_kernels.h"
 
 namespace mlstm {
 
-template <typename T, int D>
+template <typename T, int D, bool STRICT = false>
 struct ColCfg {
     // G / W tiles [query][key], written by lanes in phase A and read transposed in phase B.  16-bit: 128-byte rows,
     // 16-byte chunk c of row q stored at chunk c ^ gkey(q); fp32: rows padded by 8 floats.
@@ -27,7 +28,9 @@ struct ColCfg {
     static constexpr size_t TILE_ELEMS = (size_t)GRAN * D;
     static constexpr size_t STAGE_BYTES = 2 * TILE_ELEMS * sizeof(T) + 3 * GRAN * sizeof(float);  // Q, dH, (beta, 1/n, db)
     static constexpr size_t G_BYTES = (size_t)GRAN * LDG * sizeof(T);
-    static constexpr size_t FIXED_BYTES = 2 * G_BYTES + 2 * GRAN * sizeof(float);                  // G, W, row-sum scratch
+    // G, W (split mode: and their low-order terms), row-sum scratch.  With the two extra tiles the 16-bit D = 256 case
+    // no longer fits two query stages and runs single-staged.
+    static constexpr size_t FIXED_BYTES = (STRICT ? 4 : 2) * G_BYTES + 2 * GRAN * sizeof(float);
     static constexpr int STAGES = (2 * STAGE_BYTES + FIXED_BYTES + 2048 * sizeof(float) <= 160 * 1024) ? 2 : 1;
     static constexpr size_t LDS_BYTES = STAGES * STAGE_BYTES + FIXED_BYTES;  // plus one float per key tile, appended at launch
 };
@@ -37,11 +40,12 @@ struct ColCfg {
 // phase B gathers 4 consecutive rows x 64 bytes (rows q and q+2 land in different halves of the row).
 __device__ __forceinline__ int gkey(int q) { return (((q >> 1) & 1) << 2) | ((q >> 2) & 3); }
 
-template <typename T, int D>
+// STRICT (16-bit types): split mode, see ColArgs::precise.
+template <typename T, int D, bool STRICT>
 __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     using R = Tr<T>;
-    using Cfg = ColCfg<T, D>;
+    using Cfg = ColCfg<T, D, STRICT>;
     typedef typename R::frag frag;
     constexpr int KW = R::KW, NS = D / KW, NX = D / 64, NQS = GRAN / KW;
     // Phase B ownership.  D >= 128: wave w accumulates output column blocks {w*NXW .. } for BOTH key blocks, so each
@@ -57,7 +61,9 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
 #define ST_ROW(st) (reinterpret_cast<float*>(ST_DH(st) + Cfg::TILE_ELEMS))
     T* const Gs = reinterpret_cast<T*>(smem + STAGES * Cfg::STAGE_BYTES);
     T* const Ws = Gs + GRAN * LDG;
-    float* const rowtmp = reinterpret_cast<float*>(Ws + GRAN * LDG);  // [2][64]
+    T* const Gl = Ws + GRAN * LDG;                                    // split mode: low-order terms of G and W
+    T* const Wl = Gl + GRAN * LDG;
+    float* const rowtmp = reinterpret_cast<float*>(Gs + (STRICT ? 4 : 2) * GRAN * LDG);  // [2][64]
     float* const sG = reinterpret_cast<float*>(smem + Cfg::LDS_BYTES);  // granule bases minus this key tile's (see row kernel)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
@@ -271,8 +277,18 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                 int off;  // element offset of keys 32*kbA + 8*a4 + 4*h .. +3 of row 32*qbA + c32
                 if constexpr (R::HALF) off = (32 * qbA + c32) * GRAN + (((4 * kbA + a4) ^ gkey(c32)) << 3) + 4 * h;
                 else off = (32 * qbA + c32) * LDG + 32 * kbA + 8 * a4 + 4 * h;
-                *reinterpret_cast<typename R::vec4*>(Gs + off) = R::cvt4(gv);
-                *reinterpret_cast<typename R::vec4*>(Ws + off) = R::cvt4(wv);
+                if constexpr (STRICT) {
+                    typename R::vec4 ghi, glo, whi, wlo;
+                    R::cvt4_split(gv, ghi, glo);
+                    R::cvt4_split(wv, whi, wlo);
+                    *reinterpret_cast<typename R::vec4*>(Gs + off) = ghi;
+                    *reinterpret_cast<typename R::vec4*>(Ws + off) = whi;
+                    *reinterpret_cast<typename R::vec4*>(Gl + off) = glo;
+                    *reinterpret_cast<typename R::vec4*>(Wl + off) = wlo;
+                } else {
+                    *reinterpret_cast<typename R::vec4*>(Gs + off) = R::cvt4(gv);
+                    *reinterpret_cast<typename R::vec4*>(Ws + off) = R::cvt4(wv);
+                }
             }
             const float rs = sum_halves(rsum);
             if (h == 0) rowtmp[kbA * GRAN + 32 * qbA + c32] = rs;
@@ -286,6 +302,9 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
         if (tid < GRAN) { rp0 = rowtmp[tid]; rp1 = rowtmp[GRAN + tid]; }
         // operand fragments of contraction step t: the next step's are read while this step's MFMAs run
         frag gB[2][NKB], wB[2][NKB], qa[2][NXW], ha[2][NXW];
+        // (split mode: the low-order fragments are single-buffered, read at the start of their own step behind the
+        // MFMAs on the high-order ones: a second set of them does not fit the registers at D = 256)
+        frag gL[STRICT ? NKB : 1], wL[STRICT ? NKB : 1];
         auto read_gw = [&](int t, int kb) {
             if constexpr (R::HALF) {
                 gB[t & 1][kb] = gw_read(Gs, t, kb);
@@ -320,8 +339,15 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                         if (x == 0) read_gw(t + 1, kb);
                         if (kb == 0) read_qh(t + 1, x);
                     }
+                    if constexpr (STRICT) {
+                        if (x == 0) { gL[kb] = gw_read(Gl, t, kb); wL[kb] = gw_read(Wl, t, kb); }
+                    }
                     R::mma(dkacc[kb][x], qa[t & 1][x], gB[t & 1][kb]);
                     R::mma(dvacc[kb][x], ha[t & 1][x], wB[t & 1][kb]);
+                    if constexpr (STRICT) {
+                        R::mma(dkacc[kb][x], qa[t & 1][x], gL[kb]);
+                        R::mma(dvacc[kb][x], ha[t & 1][x], wL[kb]);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -391,19 +417,28 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
 #endif
 }
 
-template <typename T, int D>
-static int launch_col_t(const ColArgs& a, hipStream_t st) {
-    using Cfg = ColCfg<T, D>;
-    static bool attr_set = false;
-    auto kern = col_kernel<T, D>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(Cfg::LDS_BYTES + 2048 * sizeof(float)));
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+template <typename T, int D, bool STRICT>
+static int launch_col_ts(const ColArgs& a, hipStream_t st) {
+    using Cfg = ColCfg<T, D, STRICT>;
+    auto kern = col_kernel<T, D, STRICT>;
+    static std::once_flag once;
+    static hipError_t attr_rc = hipSuccess;
+    std::call_once(once, [&] {
+        attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)(Cfg::LDS_BYTES + 2048 * sizeof(float)));
+    });
+    if (attr_rc != hipSuccess) return (int)attr_rc;
+    if (a.NG > 2048) return MLSTM_ESHAPE;
     hipLaunchKernelGGL(kern, dim3(a.BH * a.NG), dim3(256), Cfg::LDS_BYTES + (size_t)a.NG * sizeof(float), st, a);
     return (int)hipGetLastError();
+}
+
+template <typename T, int D>
+static int launch_col_t(const ColArgs& a, hipStream_t st) {
+    if constexpr (Tr<T>::HALF) {
+        if (a.precise) return launch_col_ts<T, D, true>(a, st);
+    }
+    return launch_col_ts<T, D, false>(a, st);
 }
 
 template <typename T>

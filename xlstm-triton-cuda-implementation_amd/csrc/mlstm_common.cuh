@@ -54,6 +54,19 @@ template <> struct Tr<__bf16> {
         return __builtin_convertvector(x, frag);
     }
     static __device__ __forceinline__ vec4 cvt4(f32x4 x) { return __builtin_convertvector(x, vec4); }
+    // Two-term split x = hi + lo with hi = x rounded to the element type and lo = the rounded remainder: a second MFMA on
+    // lo gives the product of a weight operand about 16 significant bits instead of 8 (bf16) / 11 (fp16).
+    static __device__ __forceinline__ void from_acc_split(const f32x16& c, int t, frag& hi, frag& lo) {
+        f32x8 x;
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = c[8 * t + e];
+        hi = __builtin_convertvector(x, frag);
+        lo = __builtin_convertvector(x - __builtin_convertvector(hi, f32x8), frag);
+    }
+    static __device__ __forceinline__ void cvt4_split(f32x4 x, vec4& hi, vec4& lo) {
+        hi = __builtin_convertvector(x, vec4);
+        lo = __builtin_convertvector(x - __builtin_convertvector(hi, f32x4), vec4);
+    }
 };
 
 template <> struct Tr<_Float16> {
@@ -71,6 +84,19 @@ template <> struct Tr<_Float16> {
         return __builtin_convertvector(x, frag);
     }
     static __device__ __forceinline__ vec4 cvt4(f32x4 x) { return __builtin_convertvector(x, vec4); }
+    // Two-term split x = hi + lo with hi = x rounded to the element type and lo = the rounded remainder: a second MFMA on
+    // lo gives the product of a weight operand about 16 significant bits instead of 8 (bf16) / 11 (fp16).
+    static __device__ __forceinline__ void from_acc_split(const f32x16& c, int t, frag& hi, frag& lo) {
+        f32x8 x;
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = c[8 * t + e];
+        hi = __builtin_convertvector(x, frag);
+        lo = __builtin_convertvector(x - __builtin_convertvector(hi, f32x8), frag);
+    }
+    static __device__ __forceinline__ void cvt4_split(f32x4 x, vec4& hi, vec4& lo) {
+        hi = __builtin_convertvector(x, vec4);
+        lo = __builtin_convertvector(x - __builtin_convertvector(hi, f32x4), vec4);
+    }
 };
 
 template <> struct Tr<float> {
@@ -89,6 +115,9 @@ template <> struct Tr<float> {
         return x;
     }
     static __device__ __forceinline__ vec4 cvt4(f32x4 x) { return x; }
+    // (fp32 operands are exact: there is no split mode; these keep the shared templates well-formed)
+    static __device__ __forceinline__ void from_acc_split(const f32x16& c, int t, frag& hi, frag& lo) { hi = from_acc(c, t); lo = frag{0.f, 0.f, 0.f, 0.f}; }
+    static __device__ __forceinline__ void cvt4_split(f32x4 x, vec4& hi, vec4& lo) { hi = x; lo = vec4{0.f, 0.f, 0.f, 0.f}; }
 };
 
 // Output gate of the scan form (mlstm_scan.py:277): silu(o) * h on four packed elements, in fp32.
@@ -491,15 +520,27 @@ template <typename T> __device__ __forceinline__ float to_f32(T x) { return (flo
 //   n = max(|b|, exp(-m)) + 1e-6,  dn = -(dh . h) / n,  db = sign(b) dn [|b| > exp(-m)].
 // The reference obtains dn from a full tile loop (mlstm_matmul_kernel_backward_db, mlstm_matmul.py:133-197); because
 // sum_j C~_ij (dh_i . v_j) = n_i (dh_i . h_i) it collapses to one dot product per row.
+// hrow_lo (may be null): the remainder h - (h rounded to the element type), left by a forward in split mode; with it
+// the dot product sees h to about 16 significant bits.
 template <typename T, int NS>
 __device__ __forceinline__ void row_stats(const typename Tr<T>::frag (&xf)[NS], const T* hrow, int h, float b, float m, float& inv_n,
-                                          float& db) {
+                                          float& db, const T* hrow_lo = nullptr) {
     float acc = 0.f;
 #pragma unroll
     for (int s = 0; s < NS; s++) {
         const typename Tr<T>::frag hf = frag_rowmajor<T>(hrow, s, h);
 #pragma unroll
         for (int e = 0; e < Tr<T>::EPL; e++) acc += (float)xf[s][e] * (float)hf[e];
+    }
+    if (hrow_lo) {
+        float acc_lo = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const typename Tr<T>::frag hf = frag_rowmajor<T>(hrow_lo, s, h);
+#pragma unroll
+            for (int e = 0; e < Tr<T>::EPL; e++) acc_lo += (float)xf[s][e] * (float)hf[e];
+        }
+        acc += acc_lo;
     }
     const float delta = sum_halves(acc);
     const float em = __expf(-m);

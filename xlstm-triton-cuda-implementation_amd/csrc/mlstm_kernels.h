@@ -49,13 +49,19 @@ struct RowArgs {
     float* inv_n;
     float* db;
     int BH, S, NG;
+    // Split mode (16-bit types, generic kernel only): the weights of the second product enter it as two terms, hi + lo,
+    // each in the element type (two MFMAs per fragment), so that their rounding no longer limits the result.  The
+    // forward then also leaves h - (h rounded) in out_lo; the dQ pass reads it back through Hin_lo for dh . h.
+    int precise;
+    void* out_lo;
+    const void* Hin_lo;
 };
 // mode 0 = forward (H, b), mode 1 = dQ
 int launch_row_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);
 // eight waves (producer / consumer pairs per SIMD); 16-bit types and D in {128, 256} only
 int launch_row8_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);
 inline int launch_row_best(int mode, int dtype, int D, const RowArgs& a, hipStream_t st) {
-    if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic) {
+    if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic && !a.precise) {
         int rc = launch_row8_kernel(mode, dtype, D, a, st);
         if (rc != MLSTM_ESHAPE) return rc;  // extremely long sequences do not fit its LDS budget
     }
@@ -78,13 +84,14 @@ struct ColArgs {
     const void* Ek;          // [BH][n_states][D][D] reverse states, key-major (for dV)
     const void* Ev;          //   ... value-major (for dK)
     const float* gvec;       // [BH][n_states][D]
+    int precise;             // split mode (see RowArgs): G and W enter phase B as hi + lo
 };
 int launch_col_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
 // phase A as 16x16x32 products on two query halves, the element-wise part of the first between the MFMAs of the second;
 // 16-bit types at D = 128 and 256 only
 int launch_col16_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
 inline int launch_col_best(int dtype, int D, const ColArgs& a, hipStream_t st) {
-    if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic) {
+    if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic && !a.precise) {
         int rc = launch_col16_kernel(dtype, D, a, st);
         if (rc != MLSTM_ESHAPE) return rc;  // extremely long sequences do not fit its LDS budget
     }

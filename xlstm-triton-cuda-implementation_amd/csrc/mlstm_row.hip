@@ -15,6 +15,7 @@
 //
 // Memory pipeline: the two 64-key tiles of step j+1 are copied global->LDS by direct loads (no registers) into
 // the other of two LDS stages while step j is consumed; one barrier per step.  Tiles are XOR-swizzled.
+#include <mutex>
 #include <type_traits>
 #include "mlstm_common.cuh"
 #include "mlstm_kernels.h"
@@ -32,7 +33,8 @@ struct RowCfg {
     // plus one double per key tile of the head (the granule bases), appended at launch
 };
 
-template <typename T, int D, int MODE>
+// STRICT (16-bit types): split mode, see RowArgs::precise.
+template <typename T, int D, int MODE, bool STRICT>
 __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     using R = Tr<T>;
@@ -78,7 +80,9 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     float crow_base = -0.5f * __log2f((float)D) - a.beta2[poff + rowc];
     float inv_n = 0.f, dbv = 0.f;
     if constexpr (MODE == MODE_DQ) {
-        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + (hoff + rowc) * D, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv);
+        const T* hlo = nullptr;
+        if constexpr (STRICT) { if (a.Hin_lo) hlo = reinterpret_cast<const T*>(a.Hin_lo) + (hoff + rowc) * D; }
+        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + (hoff + rowc) * D, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv, hlo);
         if (row < S && h == 0) { a.inv_n[poff + row] = inv_n; a.db[poff + row] = dbv; }
     }
 #pragma unroll
@@ -198,7 +202,9 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
 #pragma unroll
         for (int t = 0; t < NSTEP32; t++) {
             hook(kb * NSTEP32 + t, 2 * NSTEP32);
-            const frag pf = R::from_acc(sacc, t);
+            frag pf, pl;
+            if constexpr (STRICT) R::from_acc_split(sacc, t, pf, pl);
+            else pf = R::from_acc(sacc, t);
             frag vf[NDB];
 #pragma unroll
             for (int d = 0; d < NDB; d++) {
@@ -206,7 +212,10 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
                 else vf[d] = swz_frag_transposed<T, D>(y2, 32 * kb + KW * t, 32 * d, lane);
             }
 #pragma unroll
-            for (int d = 0; d < NDB; d++) R::mma(oacc[d], vf[d], pf);
+            for (int d = 0; d < NDB; d++) {
+                R::mma(oacc[d], vf[d], pf);
+                if constexpr (STRICT) R::mma(oacc[d], vf[d], pl);
+            }
         }
     };
 
@@ -270,7 +279,12 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
         frag vf[2][NDB];
 #pragma unroll
         for (int d = 0; d < NDB; d++) vf[0][d] = vrd.read(y2, 0, d);
-        frag pf = R::from_acc(s0, 0);
+        frag pf, pl;
+        auto take_p = [&](const f32x16& sacc, int t) {
+            if constexpr (STRICT) R::from_acc_split(sacc, t, pf, pl);
+            else pf = R::from_acc(sacc, t);
+        };
+        take_p(s0, 0);
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             hook2(g, 4);
@@ -278,15 +292,16 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
             for (int d = 0; d < NDB; d++) {
                 if (g + 1 < 4) vf[(g + 1) & 1][d] = vrd.read(y2, KW * (g + 1), d);
                 R::mma(oacc[d], vf[g & 1][d], pf);
+                if constexpr (STRICT) R::mma(oacc[d], vf[g & 1][d], pl);
                 if (g < 2) {
 #pragma unroll
                     for (int r = (g * NDB + d) * 16 / (2 * NDB); r < (g * NDB + d + 1) * 16 / (2 * NDB); r++) weigh_reg(s1, r, ek1, er1, blk1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (g == 0) pf = R::from_acc(s0, 1);
-            if (g == 1) pf = R::from_acc(s1, 0);
-            if (g == 2) pf = R::from_acc(s1, 1);
+            if (g == 0) take_p(s0, 1);
+            if (g == 1) take_p(s1, 0);
+            if (g == 2) take_p(s1, 1);
         }
         if constexpr (MODE == MODE_FWD) bsum += blk0 * er0 + blk1 * er1;
       }
@@ -398,7 +413,14 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
                 f32x4 v;
 #pragma unroll
                 for (int c = 0; c < 4; c++) v[c] = oacc[d][4 * a4 + c] * onorm;
-                *reinterpret_cast<typename R::vec4*>(out + 32 * d + 8 * a4 + 4 * h) = R::cvt4(v);
+                if constexpr (STRICT && MODE == MODE_FWD) {
+                    typename R::vec4 hi, lo;
+                    R::cvt4_split(v, hi, lo);
+                    *reinterpret_cast<typename R::vec4*>(out + 32 * d + 8 * a4 + 4 * h) = hi;
+                    if (a.out_lo) *reinterpret_cast<typename R::vec4*>(reinterpret_cast<T*>(a.out_lo) + (hoff + row) * D + 32 * d + 8 * a4 + 4 * h) = lo;
+                } else {
+                    *reinterpret_cast<typename R::vec4*>(out + 32 * d + 8 * a4 + 4 * h) = R::cvt4(v);
+                }
             }
         if constexpr (MODE == MODE_FWD) {
             if (a.O) {  // gated copy from the fp32 accumulators
@@ -421,20 +443,28 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
 #endif
 }
 
-template <typename T, int D, int MODE>
-static int launch_row_t(const RowArgs& a, hipStream_t st) {
+template <typename T, int D, int MODE, bool STRICT>
+static int launch_row_ts(const RowArgs& a, hipStream_t st) {
     using Cfg = RowCfg<T, D>;
-    static bool attr_set = false;
-    auto kern = row_kernel<T, D, MODE>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(Cfg::STAGES_BYTES + 2048 * sizeof(double)));
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    auto kern = row_kernel<T, D, MODE, STRICT>;
+    static std::once_flag once;
+    static hipError_t attr_rc = hipSuccess;
+    std::call_once(once, [&] {
+        attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      (int)(Cfg::STAGES_BYTES + 2048 * sizeof(double)));
+    });
+    if (attr_rc != hipSuccess) return (int)attr_rc;
     const int nQT = (a.S + ROW_BQ - 1) / ROW_BQ;
     hipLaunchKernelGGL(kern, dim3(a.BH * nQT), dim3(256), Cfg::STAGES_BYTES + (size_t)a.NG * sizeof(double), st, a);
     return (int)hipGetLastError();
+}
+
+template <typename T, int D, int MODE>
+static int launch_row_t(const RowArgs& a, hipStream_t st) {
+    if constexpr (Tr<T>::HALF) {
+        if (a.precise) return launch_row_ts<T, D, MODE, true>(a, st);
+    }
+    return launch_row_ts<T, D, MODE, false>(a, st);
 }
 
 template <typename T, int MODE>

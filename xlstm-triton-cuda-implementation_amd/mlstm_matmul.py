@@ -11,7 +11,7 @@ import torch
 from . import _ffi
 
 
-def _check_inputs(q, k, v, f, i):
+def _check_inputs(q, k, v, f, i, precise=False):
     if q.dim() != 4:
         raise ValueError(f"q must be [B, NH, S, D], got {tuple(q.shape)}")
     B, NH, S, D = q.shape
@@ -24,12 +24,12 @@ def _check_inputs(q, k, v, f, i):
         raise TypeError("q, k, v must share one dtype")
     if i.dtype != f.dtype:
         raise TypeError("f and i must share one dtype")
-    return B, NH, S, D, _ffi.dtype_code(q.dtype), _ffi.dtype_code(f.dtype)
+    return B, NH, S, D, _ffi.dtype_code(q.dtype, precise), _ffi.dtype_code(f.dtype)
 
 
-def mlstm_forward_hip(q, k, v, f, i):
+def mlstm_forward_hip(q, k, v, f, i, precise=False):
     """Returns (h, m, b): h [B,NH,S,D] in q's dtype, m and b [B,NH,S] fp32 (reference mlstm_matmul.py:373-378)."""
-    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     h = torch.empty_like(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     b = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
@@ -40,10 +40,10 @@ def mlstm_forward_hip(q, k, v, f, i):
     return h, m, b
 
 
-def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None):
+def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False):
     """Returns (dq, dk, dv, df, di) (reference mlstm_matmul.py:384-405).  h, m, b: the forward's outputs, or None
     to have them recomputed."""
-    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     _ffi.require(dh, "dh", q.shape)
     if dh.dtype != q.dtype:
         raise TypeError("dh must have q's dtype")
@@ -59,10 +59,10 @@ def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None):
     return dq, dk, dv, df, di
 
 
-def mlstm_forward_save_hip(q, k, v, f, i):
+def mlstm_forward_save_hip(q, k, v, f, i, precise=False):
     """Forward of a training step.  Returns (h, m, b, saved): as mlstm_forward_hip, plus what the backward can reuse (the
     states at the chunk ends of a long 16-bit sequence; None for shapes that do not run in chunks)."""
-    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     h = torch.empty_like(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     b = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
@@ -76,9 +76,9 @@ def mlstm_forward_save_hip(q, k, v, f, i):
     return h, m, b, saved
 
 
-def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved):
+def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=False):
     """Backward of a training step with the forward's outputs and its saved states (mlstm_forward_save_hip)."""
-    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     _ffi.require(dh, "dh", q.shape)
     if dh.dtype != q.dtype:
         raise TypeError("dh must have q's dtype")
@@ -117,6 +117,27 @@ class Triton_mLSTM(torch.autograd.Function):
 
 
 HIP_mLSTM = Triton_mLSTM
+
+
+class Triton_mLSTM_precise(torch.autograd.Function):
+    """Triton_mLSTM in split mode (no counterpart in the reference, whose kernels are fp32): for fp16 / bf16 inputs the
+    weights of every second product enter it as two terms, so that results and gradients agree with an fp32
+    evaluation of the reference's formulas element by element at rtol 2e-2 / atol 2e-3.  Slower: no chunking, half as
+    many MFMAs again.  Same call signature."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, f, i, SB=16, num_warps=8):
+        h, m, b, saved = mlstm_forward_save_hip(q, k, v, f, i, precise=True)
+        ctx.save_for_backward(q, k, v, f, i, m, b, h, saved)
+        ctx.sb = SB
+        return h
+
+    @staticmethod
+    def backward(ctx, dh):
+        assert dh.is_contiguous()
+        q, k, v, f, i, m, b, h, saved = ctx.saved_tensors
+        dq, dk, dv, df, di = mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=True)
+        return dq, dk, dv, df, di, None, None
 
 
 # ---------------------------------------------------------------------------------------------------------------
