@@ -112,6 +112,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (torch) before the steps: under rocprofv3 --pmc its "
                          "FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
@@ -139,7 +140,8 @@ def main():
     h, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
     m, b = (torch.empty((B, NH, S), device=dev, dtype=torch.float32) for _ in range(2))
     df, di = torch.empty_like(f), torch.empty_like(i)
-    dt_code = ffi.dtype_code(dtype)
+    dt_code = ffi.dtype_code(dtype, args.precise)
+    gate_code = ffi.dtype_code(dtype)
     ws, ws_n = ffi.workspace(ffi.OP_BACKWARD, B, NH, S, D, dt_code, dev)
     st = ffi.stream_ptr()
     P = ffi.ptr
@@ -150,11 +152,11 @@ def main():
     saved = torch.empty(max(nsaved, 1), dtype=torch.uint8, device=dev)
 
     def step():
-        rc = L.mlstm_forward_save_ex(P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, B, NH, S, D, dt_code, dt_code,
+        rc = L.mlstm_forward_save_ex(P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, B, NH, S, D, dt_code, gate_code,
                                      P(ws), ws_n, st)
         ffi.check_rc(rc, "mlstm_forward_save_ex")
         rc = L.mlstm_backward_saved_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, P(dq), P(dk), P(dv),
-                                       P(df), P(di), B, NH, S, D, dt_code, dt_code, P(ws), ws_n, st)
+                                       P(df), P(di), B, NH, S, D, dt_code, gate_code, P(ws), ws_n, st)
         ffi.check_rc(rc, "mlstm_backward_saved_ex")
 
     if args.calibrate_copy:
