@@ -2,9 +2,12 @@
  * libmlstm_hip.so -- C ABI of the MI355X (gfx950) mLSTM kernels.
  *
  * Every pointer is caller-owned DEVICE memory, row-major contiguous; the library never frees or keeps it.
- * Calls are asynchronous on the given HIP stream (NULL = the default stream), re-entrant, and return 0 on
- * success, a positive hipError_t on a runtime failure, or a negative MLSTM_E* code for a rejected argument.
- * They never abort and never throw.  Shapes: q, k, v, h, dh, o and their gradients are [B, NH, S, D];
+ * Calls are asynchronous on the given HIP stream (NULL = the default stream) and return 0 on success, a positive
+ * hipError_t on a runtime failure, or a negative MLSTM_E* code for a rejected argument.  They never abort and never
+ * throw.  The compute entry points may be called from several threads at once (on different streams and buffers);
+ * the process-wide settings further down (timing, chunk length, generic kernels, spin limit) are test and
+ * measurement aids: they are not synchronised with calls in flight and must not change between a forward and the
+ * backward that reads its `saved` buffer.  Shapes: q, k, v, h, dh, o and their gradients are [B, NH, S, D];
  * f, i, m, b and their gradients are [B, NH, S].
  *
  * Each entry point names the interface of the reference it replaces (paths relative to the reference
@@ -39,6 +42,7 @@ extern "C" {
 #define MLSTM_EINVAL (-1)      /* null pointer, non-positive size, unknown dtype */
 #define MLSTM_ESHAPE (-2)      /* head dimension / sequence length not supported by this build */
 #define MLSTM_EWORKSPACE (-3)  /* caller workspace smaller than mlstm_workspace_bytes() */
+#define MLSTM_EKERNEL (-4)     /* a kernel's bounded wait expired (mlstm_kernel_error) */
 
 /* operations, for mlstm_workspace_bytes */
 #define MLSTM_OP_FORWARD 0
@@ -106,8 +110,9 @@ int mlstm_backward_ex(const void* dh, const void* q, const void* k, const void* 
  * backward with ctx.save_for_backward (mlstm_matmul.py:379: q, k, v, f, i, m, b), plus, for sequences that run in
  * chunks, the states at the chunk ends and the gate pre-pass, so that the backward does not form them again.  `saved` is caller-owned device
  * memory of mlstm_saved_state_bytes(...) bytes (0 for shapes that do not run in chunks: saved may then be NULL), written
- * by mlstm_forward_save_ex and read by mlstm_backward_saved_ex for the same inputs; the chunk length
- * (mlstm_set_chunk_length) must not change in between.  Otherwise as mlstm_forward_ex / mlstm_backward_ex, with h, m
+ * by mlstm_forward_save_ex and read by mlstm_backward_saved_ex for the same inputs and the same dtype argument; the
+ * chunk length (mlstm_set_chunk_length) must not change in between (saved_bytes must equal mlstm_saved_state_bytes
+ * at the time of either call, which catches a change of the number of chunks).  Otherwise as mlstm_forward_ex / mlstm_backward_ex, with h, m
  * and b required in the backward.  MLSTM_EWORKSPACE also reports a `saved` buffer that is missing or too small.
  */
 size_t mlstm_saved_state_bytes(int B, int NH, int S, int D, int dtype);
@@ -162,7 +167,6 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype);
  */
 #define MLSTM_K_GATES 0     /* gate pre-pass */
 #define MLSTM_K_ROW_FWD 1   /* forward tile kernel (H, b) */
-#define MLSTM_K_ROWSTATS 2  /* unused: the per-row n, db are computed inside the dQ kernel */
 #define MLSTM_K_COL 3       /* backward tile kernel (dK, dV, dI, row partials) */
 #define MLSTM_K_ROW_DQ 4    /* backward tile kernel (dQ) */
 #define MLSTM_K_DF 5        /* row reduce + dF scan */
@@ -199,6 +203,18 @@ int mlstm_set_chunk_length(int length);
 /* The chunk length the entry points use for this shape under the current setting, 0 = the sequence is not cut
  * (measurement aid: the work a chunked kernel executes depends on it). */
 int mlstm_chunk_length_for(int S, int D, int dtype);
+
+/*
+ * Fail-safe of the eight-wave row kernel, no counterpart in the reference.  Inside a workgroup its producer waves wait
+ * for an LDS counter before they reuse a buffer; the wait is bounded, and if it ever expires (a bug: it cannot in a
+ * correct build) the kernel sets a per-GPU error word and runs on to its end instead of hanging the GPU.
+ * mlstm_kernel_error waits for the current device's work, returns MLSTM_EKERNEL if the word is set (results since the
+ * last call are then not to be trusted) and clears it, 0 otherwise.  mlstm_set_spin_limit is the test aid for it:
+ * limit > 0 replaces the bound (loop iterations), limit < 0 makes every such wait count as expired without waiting
+ * (the results of that run are undefined), 0 restores the default.  Process-wide.
+ */
+int mlstm_kernel_error(void);
+int mlstm_set_spin_limit(int limit);
 
 /* Library version string, e.g. "mlstm_hip 0.1 gfx950". */
 const char* mlstm_version(void);

@@ -14,7 +14,8 @@ NOALLOC_MAX_WORKSPACE = 8 << 20   # MLSTM_NOALLOC_MAX_WORKSPACE
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dtype)",
            -2: "unsupported shape (head dimension / sequence length)",
-           -3: "workspace too small"}
+           -3: "workspace (or saved buffer) too small or of the wrong size",
+           -4: "a kernel's bounded wait expired"}
 
 _lib = None
 
@@ -62,6 +63,10 @@ def lib():
         L.mlstm_set_chunk_length.argtypes = [ci]
         L.mlstm_chunk_length_for.restype = ci
         L.mlstm_chunk_length_for.argtypes = [ci] * 3
+        L.mlstm_kernel_error.restype = ci
+        L.mlstm_kernel_error.argtypes = []
+        L.mlstm_set_spin_limit.restype = ci
+        L.mlstm_set_spin_limit.argtypes = [ci]
         L.mlstm_force_generic_kernels.restype = ci
         L.mlstm_force_generic_kernels.argtypes = [ci]
         L.mlstm_timing_read.restype = ci
@@ -75,10 +80,10 @@ def exported_symbols():
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
-            "mlstm_force_generic_kernels"]
+            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit"]
 
 
-KERNELS = {"gates": 0, "row_fwd": 1, "rowstats": 2, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
+KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
            "scan_out": 8, "gate_bwd": 9, "chunk_states": 10}
 
 

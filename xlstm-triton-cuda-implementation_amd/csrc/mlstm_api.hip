@@ -95,7 +95,7 @@ struct Sizes {
 };
 
 // begin/end marks for groups of scan kernels (the scan translation unit has no access to Timed)
-Timed* g_scan_mark[16] = {};
+thread_local Timed* g_scan_mark[16] = {};
 void scan_mark(int id, hipStream_t st, bool begin) {
     if (begin) g_scan_mark[id] = new Timed(id, st);
     else { delete g_scan_mark[id]; g_scan_mark[id] = nullptr; }
@@ -134,23 +134,38 @@ struct Scratch {
 // per device (with that device current) and everything after that -- kernel arguments included -- uses the pointer.
 constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)MLSTM_NOALLOC_MAX_WORKSPACE;
 static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+// Error word of the kernels' bounded waits (mlstm_kernel_error): one int per GPU, zero when the library is loaded, only
+// ever or-ed into by kernels and cleared by mlstm_kernel_error.
+static __device__ int kernel_error_word;
 constexpr int NOALLOC_MAX_DEVICES = 64;
 void* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+int* g_err_ptr[NOALLOC_MAX_DEVICES] = {};
 std::mutex g_scratch_mu;
-int scratch_of_current_device(char** out) {
+int symbols_of_current_device(char** scratch_out, int** err_out) {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return (int)e;
     if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return MLSTM_EINVAL;
     std::lock_guard<std::mutex> lk(g_scratch_mu);
     if (!g_scratch_ptr[dev]) {
-        void* p = nullptr;
+        void *p = nullptr, *pe = nullptr;
         e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e == hipSuccess) e = hipGetSymbolAddress(&pe, HIP_SYMBOL(kernel_error_word));
         if (e != hipSuccess) return (int)e;
-        if (!p) return (int)hipErrorInvalidSymbol;
+        if (!p || !pe) return (int)hipErrorInvalidSymbol;
         g_scratch_ptr[dev] = p;
+        g_err_ptr[dev] = static_cast<int*>(pe);
     }
-    *out = static_cast<char*>(g_scratch_ptr[dev]);
+    if (scratch_out) *scratch_out = static_cast<char*>(g_scratch_ptr[dev]);
+    if (err_out) *err_out = g_err_ptr[dev];
+    return 0;
+}
+int g_spin_limit = 0;   // test aid (mlstm_set_spin_limit): 0 = the default bound
+constexpr int DEFAULT_SPIN_LIMIT = 1 << 22;   // iterations of 64 cycles and an LDS read each: a fraction of a second
+// error word and wait bound of the eight-wave row kernel
+int arm_row_args(RowArgs& a) {
+    if (int rc = symbols_of_current_device(nullptr, &a.err)) return rc;
+    a.spin_limit = g_spin_limit == 0 ? DEFAULT_SPIN_LIMIT : g_spin_limit;
     return 0;
 }
 
@@ -214,6 +229,7 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
     a.ek2 = ek2; a.amax2 = amax2; a.O = o; a.out_gated = h_gated;
     a.BH = (int)z.BH; a.S = (int)z.S; a.NG = (int)z.NG;
     a.precise = z.precise ? 1 : 0; a.out_lo = h_lo;
+    if (int rc = arm_row_args(a)) return rc;
     if (ncs > 0) {   // long sequence: the states at the chunk ends first, then every row tile stays inside its chunk
         float* Nst = Nst_ext ? Nst_ext : w.Nst;
         if (int e = chunk_states_impl(k, v, w, true, CstT, Nst, z, D, dtype, st)) return e;
@@ -248,6 +264,26 @@ int mlstm_chunk_length_for(int S, int D, int dtype) {
 int mlstm_set_chunk_length(int length) {
     if (length > 0 && length % 128 != 0) return MLSTM_EINVAL;
     g_chunk_override = length;
+    return 0;
+}
+
+int mlstm_set_spin_limit(int limit) {
+    g_spin_limit = limit;
+    return 0;
+}
+
+int mlstm_kernel_error(void) {
+    int* word = nullptr;
+    if (int rc = symbols_of_current_device(nullptr, &word)) return rc;
+    int value = 0;
+    hipError_t e = hipMemcpy(&value, word, sizeof(int), hipMemcpyDeviceToHost);   // (waits for the device's work)
+    if (e != hipSuccess) return (int)e;
+    if (value != 0) {
+        const int zero = 0;
+        e = hipMemcpy(word, &zero, sizeof(int), hipMemcpyHostToDevice);
+        if (e != hipSuccess) return (int)e;
+        return MLSTM_EKERNEL;
+    }
     return 0;
 }
 
@@ -326,7 +362,7 @@ int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const 
     const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
     if (z.fwd() > NOALLOC_SCRATCH_BYTES) return MLSTM_EWORKSPACE;   // the shape needs more scratch than the array holds
     char* ws = nullptr;
-    if (int rc = scratch_of_current_device(&ws)) return rc;
+    if (int rc = symbols_of_current_device(&ws, nullptr)) return rc;
     // Nothing in the workspace has to start at zero: the gate pre-pass writes every element the tile kernels read,
     // padding included, and the states are written before they are read; what the previous call left is overwritten.
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, ws, st);
@@ -348,7 +384,7 @@ int mlstm_forward_save_ex(const void* q, const void* k, const void* v, const voi
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (z.saved() > 0 && (!saved || saved_bytes < z.saved())) return MLSTM_EWORKSPACE;
+    if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     char* sv = z.saved() > 0 ? (char*)saved : nullptr;
@@ -441,6 +477,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ra.ek2 = ek2; ra.amax2 = amax2; ra.Hin = h; ra.Bin = bb; ra.M = mm;
     ra.BH = (int)z.BH; ra.S = (int)z.S; ra.NG = (int)z.NG;
     ra.precise = z.precise ? 1 : 0; ra.Hin_lo = h_lo;
+    if (int rc = arm_row_args(ra)) return rc;
     if (w.ncs > 0) { ra.chunk_len = w.L; ra.n_states = (int)w.ncs; ra.Cst = CstT; ra.Nst = Nst; ra.Qrow = q; ra.rowinter = rowinter; }
     {
         Timed t(MLSTM_K_ROW_DQ, st);
@@ -503,7 +540,7 @@ int mlstm_backward_saved_ex(const void* dh, const void* q, const void* k, const 
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (z.saved() > 0 && (!saved || saved_bytes < z.saved())) return MLSTM_EWORKSPACE;
+    if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;
     return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, z, D, dtype, gate_dtype, (char*)sc.p, st,

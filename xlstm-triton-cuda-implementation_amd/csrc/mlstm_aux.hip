@@ -3,7 +3,7 @@
 //   rowreduce_kernel: x_t = col_t - sum_J rowpart[J][t]  and dI = col  (mlstm_matmul.py:309,316).
 //   dfscan_kernel   : dF_t = sigmoid(-f_t) * sum_{s<t} x_s, dF_0 = 0  (mlstm_matmul_kernel_df,
 //                     mlstm_matmul.py:320-333): wave64 DPP scans, LDS carry across waves, fp64 carry across blocks.
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {

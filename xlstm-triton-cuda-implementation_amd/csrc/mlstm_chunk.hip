@@ -15,7 +15,7 @@
 //   chunk_carry_kernel  C~_c = gamma_c C~_{c-1} + dC_c over the chunks of a head (gamma_c = exp(A_{e_{c-1}} - A_{e_c})),
 //                       element-wise, written in the element type; n~_c likewise, in place, fp32.
 // State rows are stored in the order in which the row kernel's second product contracts them (see PERM16 below).
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 #include <type_traits>
 
@@ -330,13 +330,8 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
 template <typename T, int D>
 static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     using Cfg = ChunkCfg<T, D>;
-    static bool attr_set = false;
     auto kern = chunk_sum_kernel<T, D>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D>>(160 * 1024); e != hipSuccess) return (int)e;
     if (a.L > Cfg::MAX_L) return MLSTM_ESHAPE;
     hipLaunchKernelGGL(kern, dim3(a.BH * a.NCS * (D / Cfg::VW)), dim3(256), Cfg::TILE_BYTES + 2 * (size_t)a.L * sizeof(float), st, a);
     // one carry kernel: the value-major one writes both layouts and the vector states

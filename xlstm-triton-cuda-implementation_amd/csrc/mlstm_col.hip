@@ -15,7 +15,7 @@
 // and the cancellation in dF = sigmoid(-f) * cumsum(col - row) stays exact to fp32 round-off.
 #include <mutex>
 #include <type_traits>
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {

@@ -10,7 +10,7 @@
 // [2 query halves of 16].  16x16x32 operand layout: A row (key) = lane % 16, contraction elements 8*(lane/16)..+7;
 // B column (query) = lane % 16, same contraction elements; C column (query) = lane % 16, rows (keys) 4*(lane/16) + r.
 #include <type_traits>
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {
@@ -639,14 +639,8 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 template <typename T, int D>
 static int launch_col16_t(const ColArgs& a, hipStream_t st) {
     using Cfg = Col16Cfg<T, D>;
-    static bool attr_set = false;
     auto kern = col16_kernel<T, D>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           (int)(Cfg::LDS_BYTES + 2048 * sizeof(float)));
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    if (hipError_t e = lds_limit_once<col16_kernel<T, D>>((int)(Cfg::LDS_BYTES + 2048 * sizeof(float))); e != hipSuccess) return (int)e;
     if (a.NG > 2048) return MLSTM_ESHAPE;
     hipLaunchKernelGGL(kern, dim3(a.BH * a.NG), dim3(256), Cfg::LDS_BYTES + (size_t)a.NG * sizeof(float), st, a);
     return (int)hipGetLastError();

@@ -12,7 +12,7 @@
 // whence  a_j - A_i = alpha_j - beta_i + (G_g(i) - G_g(j))  with one fp64 subtraction per tile pair.
 // alpha, beta and G are stored pre-multiplied by log2(e) (the kernels use exp2); m in natural units.
 // alpha and beta have a row stride of ceil(S/64)*64 per head (padded to whole granules).
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {

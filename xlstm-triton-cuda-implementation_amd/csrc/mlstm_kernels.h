@@ -7,6 +7,14 @@
 namespace mlstm {
 
 inline size_t dtype_size(int dt) { return dt == MLSTM_F32 ? 4 : 2; }
+
+// Raises a kernel's dynamic LDS limit, once per process and kernel; the initialisation of a function-local static is
+// thread-safe, so concurrent first calls do not race.  Returns the status of that one call.
+template <auto KERN>
+inline hipError_t lds_limit_once(int bytes) {
+    static const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    return rc;
+}
 constexpr int GATE_GRANULE = 64;  // positions per gate granule (== mlstm::GRAN in the device code)
 
 // Gate pre-pass: alpha2, beta2 [BH, NG*64] fp32 (NG = ceil(S/64), rows padded), G2 [BH, NG] fp64, M [BH,S] fp32.
@@ -55,6 +63,10 @@ struct RowArgs {
     int precise;
     void* out_lo;
     const void* Hin_lo;
+    // eight-wave kernel: the producers' wait for their P buffer is bounded; a wait that expires sets *err (sticky,
+    // see mlstm_kernel_error) and the kernel runs on to its end.  spin_limit < 0 (test aid) lets every wait expire.
+    int* err;
+    int spin_limit;
 };
 // mode 0 = forward (H, b), mode 1 = dQ
 int launch_row_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);

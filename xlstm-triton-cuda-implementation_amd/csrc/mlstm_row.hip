@@ -17,7 +17,7 @@
 // the other of two LDS stages while step j is consumed; one barrier per step.  Tiles are XOR-swizzled.
 #include <mutex>
 #include <type_traits>
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {

@@ -17,7 +17,7 @@
 // MODE_FWD replaces mlstm_matmul_kernel (mlstm_matmul.py:38-101) and the CUDA kernel mlstm_forward
 // (cuda-src/mlstm_forward.cu:14-189); MODE_DQ the dQ loop of mlstm_matmul_kernel_backward (mlstm_matmul.py:239-267).
 #include <type_traits>
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 
 namespace mlstm {
@@ -233,8 +233,21 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         auto publish = [&](const f32x16& s0, const f32x16& s1, int j) {
             frag f00 = R::from_acc(s0, 0), f01 = R::from_acc(s0, 1), f10 = R::from_acc(s1, 0), f11 = R::from_acc(s1, 1);
             if (j > 0) {
+                // Bounded: the consumers bump the counter long before it is looked at here, but a miscount must not hang
+                // the GPU.  An expired wait is reported through the error word and the kernel runs on (wrong results).
                 volatile unsigned* c = pcnt + rg;
-                while (*c < 2u * (unsigned)j) __builtin_amdgcn_s_sleep(1);
+                if (a.spin_limit < 0) {   // test aid: every wait counts as expired, without waiting
+                    if (lane == 0 && j == 1) atomicOr(a.err, 1);
+                } else {
+                    int spins = 0;
+                    while (*c < 2u * (unsigned)j) {
+                        if (spins++ >= a.spin_limit) {
+                            if (lane == 0) atomicOr(a.err, 1);
+                            break;
+                        }
+                        __builtin_amdgcn_s_sleep(1);
+                    }
+                }
             }
             p_rg[(0 + 2 * kh + 0) * 64] = f00;
             p_rg[(0 + 2 * kh + 1) * 64] = f01;
@@ -618,13 +631,8 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
 template <typename T, int D, int MODE>
 static int launch_row8_t(const RowArgs& a, hipStream_t st) {
     using Cfg = Row8Cfg<T, D>;
-    static bool attr_set = false;
     auto kern = row8_kernel<T, D, MODE>;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
-    }
+    if (hipError_t e = lds_limit_once<row8_kernel<T, D, MODE>>(160 * 1024); e != hipSuccess) return (int)e;
     const size_t lds = Cfg::FIXED_BYTES + (size_t)a.NG * sizeof(double);
     if (lds > 160 * 1024) return MLSTM_ESHAPE;  // caller falls back to the four-wave kernel
     const int nQT = (a.S + R8_BQ - 1) / R8_BQ;

@@ -17,7 +17,7 @@
 //   scan_finish_kernel  per row: b_t = decay_t (n~_{c-1} . q_t) + rowsum_t(P_c),
 //                       h = (sum of partial numerators) / (max(|b|, exp(-m)) + 1e-6) * silu(o)   (mlstm_scan.py:273-277).
 // HBM traffic: the compulsory stream of q, k, v, o, h, one round trip of the numerator per key range, q once more.
-#include "mlstm_common.cuh"
+#include "mlstm_device.h"
 #include "mlstm_kernels.h"
 #include <type_traits>
 
