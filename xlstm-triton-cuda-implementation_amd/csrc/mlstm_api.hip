@@ -77,6 +77,11 @@ struct Sizes {
     size_t states_t() const { return up256(BH * n_states(chunk_len()) * D * D * el); }   // value-major copy for the dQ pass
     size_t saved_vec() const { return up256(BH * n_states(chunk_len()) * D * 4); }
     size_t h_lo() const { return precise ? up256(BH * S * D * el) : 0; }
+    // the column kernel runs in chunks too when it is the 16x16 one (the generic kernels know no chunks), and only for
+    // lengths at which the eight-wave row kernel, which leaves the far row sums, is sure to have run
+    bool col_chunks() const { return n_states(chunk_len()) > 0 && NG <= 1024; }
+    // row partials of dD per position: one per key tile at or before it, in chunks one per key tile of its own chunk
+    size_t row_slices() const { return col_chunks() ? (size_t)chunk_len() / 64 : NG; }
     // what the backward reuses of the forward: in chunks the value-major states, the vector states and the gate
     // pre-pass; in split mode h - (h rounded to the element type)
     size_t saved() const { return precise ? h_lo() : (n_states(chunk_len()) ? states_t() + saved_vec() + gates() : 0); }
@@ -87,7 +92,7 @@ struct Sizes {
                + 2 * up256(BH * NG * 64 * 4) + states_t()                          // inv_n, db; transposed chunk states
                + 2 * states_t() + saved_vec() + up256(BH * S * 4)                  // reverse states (both layouts, vector); far row sums
                + up256(BH * n_states(chunk_len()) * 4)                             // dF anchors
-               + up256(BH * S * 4) + up256(BH * NG * S * 4)                        // colsum, rowpart
+               + up256(BH * S * 4) + up256(BH * row_slices() * S * 4)              // colsum, rowpart
                + h_lo();                                                           // split mode: low-order part of a recomputed h
     }
     // gated backward: the ungated upstream gradient, and (h, m, b) when the caller does not bring them
@@ -425,7 +430,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* inv_n = c.take<float>(z.BH * z.NG * 64);
     float* dbuf = c.take<float>(z.BH * z.NG * 64);
     float* colsum = c.take<float>(z.BH * z.S);
-    float* rowpart = c.take<float>(z.BH * z.NG * z.S);
+    float* rowpart = c.take<float>(z.BH * z.row_slices() * z.S);
     FwdWs w(ws, z, dtype, D);
     char* CstT = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);
     const float* Nst = w.Nst;
@@ -441,9 +446,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs);
     char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
-    // the column kernel runs in chunks too when it is the 16x16 one (the generic kernels know no chunks)
-    // (and only for lengths at which the eight-wave row kernel, which leaves rowinter, is sure to have run)
-    const bool col_chunks = w.ncs > 0 && z.NG <= 1024;
+    const bool col_chunks = z.col_chunks();
 
     float *alpha2, *beta2, *mm, *bb, *ek2, *amax2; double* G2;
     // Split mode needs h beyond the element type's precision for dh . h: either the forward left the low-order part
@@ -496,14 +499,14 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ca.Q = q; ca.K = k; ca.V = v; ca.dH = dh; ca.dK = dk; ca.dV = dv; ca.colsum = colsum; ca.rowpart = rowpart;
     ca.alpha2 = alpha2; ca.beta2 = beta2; ca.G2 = G2; ca.inv_n = inv_n; ca.db = dbuf;
     ca.BH = (int)z.BH; ca.S = (int)z.S; ca.NG = (int)z.NG;
-    ca.precise = z.precise ? 1 : 0;
+    ca.precise = z.precise ? 1 : 0; ca.RS = (int)z.row_slices();
     if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ek = Ek; ca.Ev = Ev; ca.gvec = gvec; }
     {
         Timed t(MLSTM_K_COL, st);
         if (int rc = launch_col_best(dtype, D, ca, st)) return rc;
     }
 
-    DfArgs da{f, colsum, rowpart, df, di, (int)z.BH, (int)z.S, (int)z.NG, col_chunks ? w.L : 0, rowinter, anchor, (int)w.ncs};
+    DfArgs da{f, colsum, rowpart, df, di, (int)z.BH, (int)z.S, (int)z.NG, (int)z.row_slices(), col_chunks ? w.L : 0, rowinter, anchor, (int)w.ncs};
     Timed t(MLSTM_K_DF, st);
     return launch_df(gate_dtype, da, st);
 }

@@ -12,26 +12,29 @@ namespace mlstm {
 // slices at or below the position's own tile), the four partial sums meet in LDS.
 template <typename TG>
 __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict__ colsum, float* rowpart, TG* __restrict__ dI,
-                                                        int S, int NG, int chunk_tiles, const float* __restrict__ rowinter) {
+                                                        int S, int NG, int RS, int chunk_tiles, const float* __restrict__ rowinter) {
     __shared__ float part[4][GRAN];
     const int bh = blockIdx.y, g = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = GRAN * g + lane, tc = t < S ? t : S - 1;
-    const float* rp = rowpart + (size_t)bh * NG * S + tc;
+    // in chunks the slices hold the key tiles of the position's own chunk only: slice = key tile - first tile of the chunk
+    const int j0 = chunk_tiles > 0 ? g / chunk_tiles * chunk_tiles : 0;
+    const int joff = RS == NG ? 0 : j0;
+    const float* rp = rowpart + (size_t)bh * RS * S + tc;
     float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
-    int j = (chunk_tiles > 0 ? g / chunk_tiles * chunk_tiles : 0) + wave;   // in chunks: from the first key tile of the position's chunk
+    int j = j0 + wave;
     for (; j + 12 <= g; j += 16) {  // four independent loads in flight per lane
-        r0 += rp[(size_t)j * S];
-        r1 += rp[(size_t)(j + 4) * S];
-        r2 += rp[(size_t)(j + 8) * S];
-        r3 += rp[(size_t)(j + 12) * S];
+        r0 += rp[(size_t)(j - joff) * S];
+        r1 += rp[(size_t)(j + 4 - joff) * S];
+        r2 += rp[(size_t)(j + 8 - joff) * S];
+        r3 += rp[(size_t)(j + 12 - joff) * S];
     }
-    for (; j <= g; j += 4) r0 += rp[(size_t)j * S];
+    for (; j <= g; j += 4) r0 += rp[(size_t)(j - joff) * S];
     part[wave][lane] = (r0 + r1) + (r2 + r3);
     __syncthreads();
     if (wave == 0 && t < S) {
         const float col = colsum[(size_t)bh * S + t];
         const float row = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]) + (rowinter ? rowinter[(size_t)bh * S + t] : 0.f);
-        rowpart[(size_t)bh * NG * S + t] = col - row;
+        rowpart[(size_t)bh * RS * S + t] = col - row;
         dI[(size_t)bh * S + t] = (TG)col;
     }
 }
@@ -42,10 +45,10 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict_
 // position's sum is off by some 2^-9 of its size, independently, and a plain running sum would add those up).
 template <typename TG>
 __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, const float* __restrict__ rowpart, TG* __restrict__ dF,
-                                                      int S, int NG, int chunk_len, const float* __restrict__ anchor, int n_states) {
+                                                      int S, int RS, int chunk_len, const float* __restrict__ anchor, int n_states) {
     __shared__ float wt[2][16];
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const float* x = rowpart + (size_t)bh * NG * S;
+    const float* x = rowpart + (size_t)bh * RS * S;
     double carry = 0.0;
     int par = 0;
     const int step = chunk_len > 0 && chunk_len < 1024 ? chunk_len : 1024;   // (a chunk is a multiple of 128 positions)
@@ -84,7 +87,7 @@ __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, 
 template <typename TG>
 __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F, const float* __restrict__ colsum, const float* __restrict__ rowpart,
                                                        const float* __restrict__ rowinter, const float* __restrict__ anchor,
-                                                       TG* __restrict__ dF, TG* __restrict__ dI, int S, int NG, int chunk_len, int n_states) {
+                                                       TG* __restrict__ dF, TG* __restrict__ dI, int S, int RS, int chunk_len, int n_states) {
     __shared__ float wt[16];
     const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t = c * chunk_len + tid;
@@ -92,9 +95,9 @@ __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F,
     float v = 0.f, col = 0.f, f = 0.f;
     if (live) {
         const int g = t / GRAN, g0 = c * (chunk_len / GRAN);
-        const float* rp = rowpart + (size_t)bh * NG * S + t;
+        const float* rp = rowpart + (size_t)bh * RS * S + t;     // slice = key tile - first tile of the chunk
         float row = rowinter[(size_t)bh * S + t];
-        for (int j = g0; j <= g; j++) row += rp[(size_t)j * S];
+        for (int j = g0; j <= g; j++) row += rp[(size_t)(j - g0) * S];
         col = colsum[(size_t)bh * S + t];
         f = (float)F[(size_t)bh * S + t];
         v = col - row;
@@ -124,14 +127,14 @@ template <typename TG>
 static int launch_df_t(const DfArgs& a, hipStream_t st) {
     if (a.chunk_len > 0 && a.chunk_len <= 1024) {
         hipLaunchKernelGGL(dfchunk_kernel<TG>, dim3((a.S + a.chunk_len - 1) / a.chunk_len, a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F),
-                           a.colsum, a.rowpart, a.rowinter, a.anchor, reinterpret_cast<TG*>(a.dF), reinterpret_cast<TG*>(a.dI), a.S, a.NG,
+                           a.colsum, a.rowpart, a.rowinter, a.anchor, reinterpret_cast<TG*>(a.dF), reinterpret_cast<TG*>(a.dI), a.S, a.RS,
                            a.chunk_len, a.n_states);
         return (int)hipGetLastError();
     }
     hipLaunchKernelGGL(rowreduce_kernel<TG>, dim3((a.S + GRAN - 1) / GRAN, a.BH), dim3(256), 0, st, a.colsum, const_cast<float*>(a.rowpart),
-                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr);
+                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.RS, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr);
     hipLaunchKernelGGL(dfscan_kernel<TG>, dim3(a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F), a.rowpart,
-                       reinterpret_cast<TG*>(a.dF), a.S, a.NG, a.chunk_len, a.anchor, a.n_states);
+                       reinterpret_cast<TG*>(a.dF), a.S, a.RS, a.chunk_len, a.anchor, a.n_states);
     return (int)hipGetLastError();
 }
 

@@ -352,7 +352,7 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                 }
             }
         }
-        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * NG + jt) * S + qi0 + tid] = rp0 + rp1;
+        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * a.RS + jt) * S + qi0 + tid] = rp0 + rp1;   // (RS == NG: no chunks here)
         if constexpr (STAGES == 1) {
             __syncthreads();  // single stage: everyone is done reading before the overwrite, which the next top barrier awaits
             if (it + 1 < NG) COL_DMA(it + 1, 0);

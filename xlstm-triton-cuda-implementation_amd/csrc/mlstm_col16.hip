@@ -572,7 +572,7 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
                 }
             }
         }
-        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * NG + jt) * S + qi0 + tid] = rp0 + rp1;
+        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * a.RS + (a.RS == NG ? jt : jt % a.RS)) * S + qi0 + tid] = rp0 + rp1;
     };
     // steps whose successor tile exists and is complete spread its copy over their MFMAs; the others copy in one go
     const int lim = (NGe < full_tiles ? NGe : full_tiles) - 1;   // last step index that may spread is lim - 1

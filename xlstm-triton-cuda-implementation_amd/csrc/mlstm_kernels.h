@@ -84,7 +84,9 @@ struct ColArgs {
     const void* Q; const void* K; const void* V; const void* dH;
     void* dK; void* dV;
     float* colsum;    // [BH,S] fp32 column sums of dD (= dI before the cast)
-    float* rowpart;   // [BH,NG,S] fp32 partial row sums of dD, one slice per key tile
+    float* rowpart;   // [BH,RS,S] fp32 partial row sums of dD, one slice per key tile (RS = NG), or, in chunks, per key
+                      // tile of the position's own chunk (RS = chunk_len / 64: slice = key tile modulo RS)
+    int RS;
     const float* alpha2; const float* beta2; const double* G2;
     const float* inv_n; const float* db;
     int BH, S, NG;
@@ -114,6 +116,7 @@ struct DfArgs {
     const void* F; const float* colsum; const float* rowpart;
     void* dF; void* dI;
     int BH, S, NG;
+    int RS;                  // row-partial slices per head (see ColArgs)
     // in chunks: rowpart holds the slices of the key tiles of the position's own chunk only, rowinter the rest
     int chunk_len;
     const float* rowinter;
