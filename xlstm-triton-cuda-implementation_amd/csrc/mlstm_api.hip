@@ -90,7 +90,7 @@ struct Sizes {
     size_t bwd() const {
         return fwd() + up256(BH * S * D * el)                                      // recomputed h
                + 2 * up256(BH * NG * 64 * 4) + states_t()                          // inv_n, db; transposed chunk states
-               + 2 * states_t() + saved_vec() + up256(BH * S * 4)                  // reverse states (both layouts, vector); far row sums
+               + states_t() + saved_vec() + up256(BH * S * 4)                      // reverse states (value-major, vector); far row sums
                + up256(BH * n_states(chunk_len()) * 4)                             // dF anchors
                + up256(BH * S * 4) + up256(BH * row_slices() * S * 4)              // colsum, rowpart
                + h_lo();                                                           // split mode: low-order part of a recomputed h
@@ -440,8 +440,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         Nst = reinterpret_cast<const float*>(saved + z.states_t());
         w.gates_at(const_cast<char*>(saved) + z.states_t() + z.saved_vec(), z);
     }
-    char* Ek = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);    // reverse states, key-major (dV) and value-major (dK)
-    char* Ev = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);
+    char* Ev = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);    // reverse states, value-major
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs);
@@ -491,7 +490,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         // reverse states from (Q, dH) and the dQ pass's per-row scalars (the column kernel applies them to its keys
         // itself), and the dF anchors at the chunk boundaries
         Timed t(MLSTM_K_CHUNK_STATES, st);
-        ChunkArgs ra2{q, dh, alpha2, beta2, G2, w.dC, gvec, Ek, Ev, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs, 1, inv_n, dbuf};
+        ChunkArgs ra2{q, dh, alpha2, beta2, G2, w.dC, gvec, nullptr, Ev, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs, 1, inv_n, dbuf};
         if (int e = launch_chunk_states(dtype, D, ra2, st)) return e;
         if (int e = launch_anchor(dtype, D, CstT, Ev, Nst, gvec, anchor, (int)z.BH, (int)w.ncs, st)) return e;   // (both value-major)
     }
@@ -500,7 +499,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ca.alpha2 = alpha2; ca.beta2 = beta2; ca.G2 = G2; ca.inv_n = inv_n; ca.db = dbuf;
     ca.BH = (int)z.BH; ca.S = (int)z.S; ca.NG = (int)z.NG;
     ca.precise = z.precise ? 1 : 0; ca.RS = (int)z.row_slices();
-    if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ek = Ek; ca.Ev = Ev; ca.gvec = gvec; }
+    if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ev = Ev; ca.gvec = gvec; }
     {
         Timed t(MLSTM_K_COL, st);
         if (int rc = launch_col_best(dtype, D, ca, st)) return rc;

@@ -138,10 +138,31 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
         }                                                                        \
         rvdma.issue(ST_ROW(st), (it));                                            \
     } while (0)
-    // every scalar the prologue needs, requested in one batch ahead of the copies (each dependent trip to memory costs a
-    // few thousand cycles here)
     const int chunk = a.chunk_len > 0 ? (GRAN * jt) / a.chunk_len : 0;
     const bool has_state = a.chunk_len > 0 && chunk < a.n_states;   // (uniform over the workgroup)
+    // The keys' own K and V rows go through LDS once (stage 1, which the query loop only needs from its second tile on):
+    // every wave wants all of them, as the second operand of the state phase below and as the stationary fragments of
+    // the query loop.  With a state phase ahead, stage 0 first carries the reverse state (two 64-row tiles at a time) and
+    // the first query tile follows when the state is done with; otherwise the first query tile travels right away.
+    // The copies are issued before anything else: the time to pull these bytes into the CU is what the prologue costs.
+    T* const Kt = ST_Q(1);
+    T* const Vt = ST_DH(1);
+    constexpr int NTL = D / GRAN;   // 64-row tiles of a state
+    const T* const Evc = has_state ? reinterpret_cast<const T*>(a.Ev) + ((size_t)bh * a.n_states + chunk) * D * D : nullptr;
+    if (GRAN * (jt + 1) <= S) {
+        tdma.issue(Kt, K + (size_t)GRAN * jt * D);
+        tdma.issue(Vt, V + (size_t)GRAN * jt * D);
+    } else {   // rows past the end are clamped
+        tile_dma<T, D, GRAN, 256>(Kt, K, GRAN * jt, S, tid);
+        tile_dma<T, D, GRAN, 256>(Vt, V, GRAN * jt, S, tid);
+    }
+    if (has_state) {
+        tdma.issue(ST_Q(0), Evc);
+        tdma.issue(ST_DH(0), Evc + (size_t)GRAN * D);
+    } else {
+        COL_DMA(jt, 0);
+    }
+    // every scalar the prologue needs, requested in one batch (each dependent trip to memory costs a few thousand cycles here)
     const int pe = has_state ? (chunk + 1) * a.chunk_len - 1 : 0;   // the chunk's last position
     const double gj = a.G2[(size_t)bh * a.NG + jt];
     const double g_first = tid < a.NG ? a.G2[(size_t)bh * a.NG + tid] : 0.0;
@@ -156,19 +177,6 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             akey[kb] = a.alpha2[poff + key];
         }
     }
-    // The keys' own K and V rows go through LDS once (stage 1, which the query loop only needs from its second tile on):
-    // every wave wants all of them, as the second operand of the state phase below and as the stationary fragments of
-    // the query loop.  The first query tile travels with them.
-    T* const Kt = ST_Q(1);
-    T* const Vt = ST_DH(1);
-    if (GRAN * (jt + 1) <= S) {
-        tdma.issue(Kt, K + (size_t)GRAN * jt * D);
-        tdma.issue(Vt, V + (size_t)GRAN * jt * D);
-    } else {   // rows past the end are clamped
-        tile_dma<T, D, GRAN, 256>(Kt, K, GRAN * jt, S, tid);
-        tile_dma<T, D, GRAN, 256>(Vt, V, GRAN * jt, S, tid);
-    }
-    COL_DMA(jt, 0);
     f32x16 dkacc[NKB][NXW], dvacc[NKB][NXW];
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
@@ -181,35 +189,19 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
     if constexpr (FAST_TR) trd.init(lane, BOTH_KB ? wave * NXW : 0);
 
     // ---- state phase (sequences in chunks): what the queries behind the keys' chunk contribute comes through the reverse
-    // states of the chunk, dV_j = w_j E^T k_j and dK_j = w_j (E v_j + g) with w_j = exp(a_j - A_e), e the chunk's last
-    // position.  A wave owns output columns, so it needs its own rows of the state only -- of the key-major copy for dK
-    // (row = key index, contracted over the values with V), of the value-major copy for dV (row = value index, contracted
-    // over the key index with K) -- and takes them straight from global memory as row-major fragments, a few steps
-    // ahead; the other operand is the keys' K / V rows out of LDS.  (Stored state row u holds row perm16(u).)
+    // state of the chunk, E[k][v] = sum_i rho_i / n_i q_i[k] dh_i[v] / sqrt(D):  dK_j = w_j (E v_j + g),  dV_j = w_j E^T k_j
+    // with w_j = exp(a_j - A_e), e the chunk's last position.  The state is stored once, value-major (row = value index,
+    // 16-row groups in the contraction order of the transposing reads), and streams through stage 0 as D/64 tiles of 64
+    // rows, two at a time.  A wave owns output columns: for dV those are rows of the state -- its own 32-row blocks, read
+    // row-major and contracted over the key index with K; for dK they are columns of the state, read with transposing
+    // loads from every tile and contracted over the tile's rows (values) with V.  The other operand of both products is
+    // the keys' K / V rows out of LDS.
     // colfar: k_j . dK_j of that part = the column sums of dD over those queries.
     float colfar = 0.f;   // thread tid < 64: key tid of the tile
-    constexpr int NT16 = D / KW, PD = 8;   // contraction steps; steps of state fragments in flight
-    frag ea[PD][NXW], eb[PD][NXW];
-    const T* ekrow[NXW];
-    const T* evrow[NXW];
+    constexpr int NT16 = D / KW;   // contraction steps of a whole row
     float wk[NKB];
     const float* gv = nullptr;
-    if (has_state) {
-#pragma unroll
-        for (int x = 0; x < NXW; x++) {
-            const int d = 32 * (wave * NXW + x) + c32, u = (d & ~15) | ((d & 3) | ((d & 4) << 1) | ((d & 8) >> 1));
-            ekrow[x] = reinterpret_cast<const T*>(a.Ek) + (((size_t)bh * a.n_states + chunk) * D + u) * D;
-            evrow[x] = reinterpret_cast<const T*>(a.Ev) + (((size_t)bh * a.n_states + chunk) * D + u) * D;
-        }
-#pragma unroll
-        for (int t = 0; t < PD; t++)
-#pragma unroll
-            for (int x = 0; x < NXW; x++) {
-                ea[t][x] = frag_rowmajor<T>(ekrow[x], t, h);
-                eb[t][x] = frag_rowmajor<T>(evrow[x], t, h);
-            }
-        gv = a.gvec + ((size_t)bh * a.n_states + chunk) * D;
-    }
+    if (has_state) gv = a.gvec + ((size_t)bh * a.n_states + chunk) * D;
     // granule bases minus this key tile's
     if (tid < a.NG) sG[tid] = (float)(g_first - gj);
     for (int g = tid + 256; g < a.NG; g += 256) sG[g] = (float)(a.G2[(size_t)bh * a.NG + g] - gj);
@@ -218,31 +210,60 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
         for (int kb = 0; kb < NKB; kb++) wk[kb] = fast_exp2(akey[kb] - bend + (float)(Gend - gj));   // (the keys' granule is jt)
     }
     dma_wait();
-    __syncthreads();   // K, V of the keys (and the first query tile) have landed
+    __syncthreads();   // K, V of the keys and the first state tiles (or the first query tile) have landed
     if (has_state) {
+        // the wave's own rows: column block cb holds stored rows 32 cb + c32 -> tile (32 cb) / 64, local row (32 cb) % 64 + c32
+        int own_row[NXW];
 #pragma unroll
-        for (int t = 0; t < NT16; t++) {
-            frag vB[NKB], kB[NKB];
+        for (int x = 0; x < NXW; x++) {
+            const int rl = (32 * (wave * NXW + x)) % GRAN + c32;
+            own_row[x] = (rl & ~15) | ((rl & 3) | ((rl & 4) << 1) | ((rl & 8) >> 1));
+        }
 #pragma unroll
-            for (int kb = 0; kb < NKB; kb++) {
-                vB[kb] = swz_frag_rowmajor<T, D>(Vt, 32 * kb + c32, t, h);
-                kB[kb] = swz_frag_rowmajor<T, D>(Kt, 32 * kb + c32, t, h);
+        for (int round = 0; round < (NTL + 1) / 2; round++) {
+            if (round > 0) {
+                tdma.issue(ST_Q(0), Evc + (size_t)GRAN * (2 * round) * D);
+                if (2 * round + 1 < NTL) tdma.issue(ST_DH(0), Evc + (size_t)GRAN * (2 * round + 1) * D);
+                dma_wait();
+                __syncthreads();
             }
 #pragma unroll
-            for (int x = 0; x < NXW; x++)
+            for (int half = 0; half < 2; half++) {
+                const int tau = 2 * round + half;
+                if (tau >= NTL) break;
+                const T* tile = half ? ST_DH(0) : ST_Q(0);
+                // dK: contraction over this tile's 64 rows (values 64 tau ..), the wave's columns of the state
 #pragma unroll
-                for (int kb = 0; kb < NKB; kb++) {
-                    R::mma(dkacc[kb][x], ea[t % PD][x], vB[kb]);
-                    R::mma(dvacc[kb][x], eb[t % PD][x], kB[kb]);
+                for (int tt = 0; tt < GRAN / KW; tt++) {
+                    const int t = (GRAN / KW) * tau + tt;
+                    frag vB[NKB], ea[NXW];
+#pragma unroll
+                    for (int kb = 0; kb < NKB; kb++) vB[kb] = swz_frag_rowmajor<T, D>(Vt, 32 * kb + c32, t, h);
+#pragma unroll
+                    for (int x = 0; x < NXW; x++) ea[x] = trd.read(tile, KW * tt, x);
+#pragma unroll
+                    for (int x = 0; x < NXW; x++)
+#pragma unroll
+                        for (int kb = 0; kb < NKB; kb++) R::mma(dkacc[kb][x], ea[x], vB[kb]);
                 }
-            if (t + PD < NT16) {
+                // dV: the wave's own rows, if this tile holds them, contracted over the whole key index
 #pragma unroll
                 for (int x = 0; x < NXW; x++) {
-                    ea[t % PD][x] = frag_rowmajor<T>(ekrow[x], t + PD, h);
-                    eb[t % PD][x] = frag_rowmajor<T>(evrow[x], t + PD, h);
+                    if ((32 * (wave * NXW + x)) / GRAN != tau) continue;
+#pragma unroll
+                    for (int t = 0; t < NT16; t++) {
+                        frag kB[NKB];
+#pragma unroll
+                        for (int kb = 0; kb < NKB; kb++) kB[kb] = swz_frag_rowmajor<T, D>(Kt, 32 * kb + c32, t, h);
+                        const frag eb = swz_frag_rowmajor<T, D>(tile, own_row[x], t, h);
+#pragma unroll
+                        for (int kb = 0; kb < NKB; kb++) R::mma(dvacc[kb][x], eb, kB[kb]);
+                    }
                 }
             }
+            __syncthreads();   // every wave is done with the two tiles
         }
+        COL_DMA(jt, 0);   // the first query tile follows the state into stage 0; it lands under the arithmetic below
         float* const cpart = reinterpret_cast<float*>(Gs);   // [4 waves][64 keys]; G / W are not in use yet
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {

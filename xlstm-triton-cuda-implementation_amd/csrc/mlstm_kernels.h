@@ -95,8 +95,7 @@ struct ColArgs {
     // written for the key tiles of the query's own chunk only
     int chunk_len;
     int n_states;
-    const void* Ek;          // [BH][n_states][D][D] reverse states, key-major (for dV)
-    const void* Ev;          //   ... value-major (for dK)
+    const void* Ev;          // [BH][n_states][D][D] reverse states, value-major (ChunkArgs::CstT of the reverse pass)
     const float* gvec;       // [BH][n_states][D]
     int precise;             // split mode (see RowArgs): G and W enter phase B as hi + lo
 };
