@@ -186,7 +186,10 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             for (int r = 0; r < 16; r++) { dkacc[kb][x][r] = 0.f; dvacc[kb][x][r] = 0.f; }
     constexpr bool FAST_TR = R::HALF && Swz<T, D>::CPR >= 16;
     SwzTransReader<typename std::conditional<FAST_TR, T, __bf16>::type, FAST_TR ? D : 256> trd;
-    if constexpr (FAST_TR) trd.init(lane, BOTH_KB ? wave * NXW : 0);
+    // Phase B column blocks of a wave: wave, wave + 4, ... (XS apart), so that its blocks are spread over the 64-row tiles of
+    // the state: with two tiles at a time in LDS every wave finds one of its own blocks in either round of the state phase
+    constexpr int XS = 4;
+    if constexpr (FAST_TR) trd.init(lane, BOTH_KB ? wave : 0);
 
     // ---- state phase (sequences in chunks): what the queries behind the keys' chunk contribute comes through the reverse
     // state of the chunk, E[k][v] = sum_i rho_i / n_i q_i[k] dh_i[v] / sqrt(D):  dK_j = w_j (E v_j + g),  dV_j = w_j E^T k_j
@@ -216,7 +219,7 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
         int own_row[NXW];
 #pragma unroll
         for (int x = 0; x < NXW; x++) {
-            const int rl = (32 * (wave * NXW + x)) % GRAN + c32;
+            const int rl = (32 * (wave + XS * x)) % GRAN + c32;
             own_row[x] = (rl & ~15) | ((rl & 3) | ((rl & 4) << 1) | ((rl & 8) >> 1));
         }
 #pragma unroll
@@ -232,38 +235,57 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
                 const int tau = 2 * round + half;
                 if (tau >= NTL) break;
                 const T* tile = half ? ST_DH(0) : ST_Q(0);
-                // dK: contraction over this tile's 64 rows (values 64 tau ..), the wave's columns of the state
+                // dK: contraction over this tile's 64 rows (values 64 tau ..), the wave's columns of the state.  Operand reads
+                // run one step ahead of the MFMAs that consume them.
+                {
+                    constexpr int NTT = GRAN / KW;
+                    frag vB[2][NKB], ea[2][NXW];
+                    auto rd = [&](int tt) {
 #pragma unroll
-                for (int tt = 0; tt < GRAN / KW; tt++) {
-                    const int t = (GRAN / KW) * tau + tt;
-                    frag vB[NKB], ea[NXW];
+                        for (int kb = 0; kb < NKB; kb++) vB[tt & 1][kb] = swz_frag_rowmajor<T, D>(Vt, 32 * kb + c32, NTT * tau + tt, h);
 #pragma unroll
-                    for (int kb = 0; kb < NKB; kb++) vB[kb] = swz_frag_rowmajor<T, D>(Vt, 32 * kb + c32, t, h);
+                        for (int x = 0; x < NXW; x++) ea[tt & 1][x] = trd.read(tile, KW * tt, XS * x);
+                    };
+                    rd(0);
 #pragma unroll
-                    for (int x = 0; x < NXW; x++) ea[x] = trd.read(tile, KW * tt, x);
+                    for (int tt = 0; tt < NTT; tt++) {
+                        if (tt + 1 < NTT) rd(tt + 1);
 #pragma unroll
-                    for (int x = 0; x < NXW; x++)
+                        for (int x = 0; x < NXW; x++)
 #pragma unroll
-                        for (int kb = 0; kb < NKB; kb++) R::mma(dkacc[kb][x], ea[x], vB[kb]);
+                            for (int kb = 0; kb < NKB; kb++) R::mma(dkacc[kb][x], ea[tt & 1][x], vB[tt & 1][kb]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
                 }
                 // dV: the wave's own rows, if this tile holds them, contracted over the whole key index
 #pragma unroll
                 for (int x = 0; x < NXW; x++) {
-                    if ((32 * (wave * NXW + x)) / GRAN != tau) continue;
+                    if ((32 * (wave + XS * x)) / GRAN != tau) continue;
+                    frag kB[2][NKB], eb[2];
+                    auto rd = [&](int t) {
+#pragma unroll
+                        for (int kb = 0; kb < NKB; kb++) kB[t & 1][kb] = swz_frag_rowmajor<T, D>(Kt, 32 * kb + c32, t, h);
+                        eb[t & 1] = swz_frag_rowmajor<T, D>(tile, own_row[x], t, h);
+                    };
+                    rd(0);
 #pragma unroll
                     for (int t = 0; t < NT16; t++) {
-                        frag kB[NKB];
+                        if (t + 1 < NT16) rd(t + 1);
 #pragma unroll
-                        for (int kb = 0; kb < NKB; kb++) kB[kb] = swz_frag_rowmajor<T, D>(Kt, 32 * kb + c32, t, h);
-                        const frag eb = swz_frag_rowmajor<T, D>(tile, own_row[x], t, h);
-#pragma unroll
-                        for (int kb = 0; kb < NKB; kb++) R::mma(dvacc[kb][x], eb, kB[kb]);
+                        for (int kb = 0; kb < NKB; kb++) R::mma(dvacc[kb][x], eb[t & 1], kB[t & 1][kb]);
+                        __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
             __syncthreads();   // every wave is done with the two tiles
         }
-        COL_DMA(jt, 0);   // the first query tile follows the state into stage 0; it lands under the arithmetic below
+        // The first query tile follows the state into stage 0.  Its copy is issued a block at a time between the pieces of
+        // the arithmetic below (a wave that issues it in one go sits in the memory pipeline's queue for its whole length)
+        const bool first_full = jt < full_tiles;
+        if (first_full) rvdma.issue(ST_ROW(0), jt);
+        else COL_DMA(jt, 0);
+        constexpr int PW0 = TileDma<T, D, GRAN, 256>::PER_WAVE;
+        constexpr int PIECES = NKB * NXW * 4;     // bodies of the loop below; both tiles' blocks are dealt out over them
         float* const cpart = reinterpret_cast<float*>(Gs);   // [4 waves][64 keys]; G / W are not in use yet
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
@@ -272,7 +294,13 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             for (int x = 0; x < NXW; x++)
 #pragma unroll
                 for (int a4 = 0; a4 < 4; a4++) {
-                    const int d = 32 * (wave * NXW + x) + 8 * a4 + 4 * h;
+                    if (first_full) {
+                        const int piece = (kb * NXW + x) * 4 + a4;
+                        const int b0 = piece * 2 * PW0 / PIECES, b1 = (piece + 1) * 2 * PW0 / PIECES;   // of 2 PW0 blocks: Q then dH
+                        if (b0 < PW0) tdma.issue_range(ST_Q(0), Q + (size_t)GRAN * jt * D, b0, b1 < PW0 ? b1 : PW0);
+                        if (b1 > PW0) tdma.issue_range(ST_DH(0), dH + (size_t)GRAN * jt * D, b0 > PW0 ? b0 - PW0 : 0, b1 - PW0);
+                    }
+                    const int d = 32 * (wave + XS * x) + 8 * a4 + 4 * h;
                     const f32x4 g4v = *reinterpret_cast<const f32x4*>(gv + d);
                     const char* kp = reinterpret_cast<const char*>(Kt) + Swz<T, D>::off(32 * kb + c32, d & ~7) + (d & 7) * (int)sizeof(T);
                     const f32x4 kv = __builtin_convertvector(*reinterpret_cast<const typename R::vec4*>(kp), f32x4);
@@ -513,8 +541,8 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             wB[t & 1][kb] = gw_read(Ws, t, kb);
         };
         auto read_qh = [&](int t, int x) {
-            qa[t & 1][x] = trd.read(Qs, KW * t, x);   // reader based at column block wave*NXW
-            ha[t & 1][x] = trd.read(dHs, KW * t, x);
+            qa[t & 1][x] = trd.read(Qs, KW * t, XS * x);   // reader based at column block `wave`
+            ha[t & 1][x] = trd.read(dHs, KW * t, XS * x);
         };
         if (!skip) {
 #pragma unroll
@@ -608,14 +636,16 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 #undef ST_ROW
 
     // ---- epilogue: dK, dV.  A lane holds 4 consecutive columns of its key's row: stored directly that would be 8-byte
-    // pieces scattered over 32 rows per instruction.  Each tensor goes through an LDS tile (rows padded by 16 bytes)
-    // and leaves in 16-byte pieces, a row at a time.
+    // pieces scattered over 32 rows per instruction.  Each tensor goes through an LDS tile of its own (rows padded by 16
+    // bytes; dK in the first query stage, dV in the second: both are free once every wave is past its last phase B) and
+    // leaves in 16-byte pieces, a row at a time.
     {
         constexpr int RB = D * (int)sizeof(T) + 16, CPR = D * (int)sizeof(T) / 16, NPC = GRAN * CPR / 256;
-        char* const stage = smem;  // the Q / dH stages are free once every wave is past its last phase B
+        static_assert((size_t)GRAN * RB <= Cfg::STAGE_BYTES, "a staged output tile fits a query stage");
+        __syncthreads();
 #pragma unroll
         for (int which = 0; which < 2; which++) {
-            __syncthreads();
+            char* const stage = smem + which * Cfg::STAGE_BYTES;
 #pragma unroll
             for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
@@ -625,10 +655,14 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
                         f32x4 v;
 #pragma unroll
                         for (int c = 0; c < 4; c++) v[c] = which ? dvacc[kb][x][4 * a4 + c] : dkacc[kb][x][4 * a4 + c];
-                        const int d = 32 * (BOTH_KB ? wave * NXW + x : dsel + 2 * x) + 8 * a4 + 4 * h;
+                        const int d = 32 * (BOTH_KB ? wave + XS * x : dsel + 2 * x) + 8 * a4 + 4 * h;
                         *reinterpret_cast<typename R::vec4*>(stage + (32 * (BOTH_KB ? kb : kbB) + c32) * RB + d * (int)sizeof(T)) = R::cvt4(v);
                     }
-            __syncthreads();
+        }
+        __syncthreads();
+#pragma unroll
+        for (int which = 0; which < 2; which++) {
+            const char* const stage = smem + which * Cfg::STAGE_BYTES;
             char* const gout = reinterpret_cast<char*>(which ? a.dV : a.dK) + (hoff + (size_t)GRAN * jt) * D * sizeof(T);
 #pragma unroll
             for (int i = 0; i < NPC; i++) {
@@ -644,12 +678,13 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < 8; r++) {
+        // sum over the 16 query lanes of a DPP row: after the four shifted adds lane 15 of the row holds the total
         float v = colacc[r];
-        v += __shfl_xor(v, 1);
-        v += __shfl_xor(v, 2);
-        v += __shfl_xor(v, 4);
-        v += __shfl_xor(v, 8);
-        if (l16 == 0) rowtmp[qbA * GRAN + 32 * kbA + 16 * (r >> 2) + 4 * g4 + (r & 3)] = v;
+        v += dpp_f<0x111>(0.f, v);
+        v += dpp_f<0x112>(0.f, v);
+        v += dpp_f<0x114>(0.f, v);
+        v += dpp_f<0x118>(0.f, v);
+        if (l16 == 15) rowtmp[qbA * GRAN + 32 * kbA + 16 * (r >> 2) + 4 * g4 + (r & 3)] = v;
     }
     __syncthreads();
     if (tid < GRAN && GRAN * jt + tid < S)
