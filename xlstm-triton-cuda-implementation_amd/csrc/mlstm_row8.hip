@@ -142,6 +142,24 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             for (int s = 0; s < NS; s++) xf[r][s] = frag_rowmajor<T>(X + (size_t)rowc[r] * D, s, h);
             crow_base[r] = -0.5f * __log2f((float)D) - a.beta2[poff + rowc[r]];
         }
+        if constexpr (MODE == R8_DQ) {
+            // Per-row scalars of the backward (1/n, db: see row_stats) for row block kh of the row group.  Behind the first
+            // chunk the consumers start with the state tiles and this role would wait for them: it has the rows' dh
+            // fragments in registers already and does the dot products with h itself.  (In the first chunk, and without
+            // chunks, it is the other way round: this role heads the critical path and the consumers idle.)
+            if (chunk > 0) {
+                float inv = 0.f, dbr = 0.f;
+                const int rc = rowc[kh];
+                const T* hrow = reinterpret_cast<const T*>(a.Hin) + (hoff + rc) * D;
+                if (kh == 0) row_stats<T, NS>(xf[0], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
+                else row_stats<T, NS>(xf[1], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
+                const int row = r0 + 32 * kh + c32;
+                if (h == 0) {
+                    *reinterpret_cast<float2*>(bex + ((rg * 2 + kh) * 32 + c32) * 2) = make_float2(inv, dbr);
+                    if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
+                }
+            }
+        }
 #pragma unroll
         for (int r = 0; r < 2; r++) {
 #pragma unroll
@@ -453,9 +471,26 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             if constexpr (MODE == R8_FWD) m_pre[r] = a.M[hoff + rowc[r]];
         }
         y2_bulk(0);
-        if constexpr (MODE == R8_DQ) {
+        // The row sums of the state part need the rows' Q behind the state tiles (q_i . dQ_i): touch the lines now, so that
+        // the loads then find them in the L2 instead of waiting for HBM in the middle of the prologue.  The touched words are
+        // only "used" behind the state tiles: a use here would wait for them, and for every copy issued before them.
+        int touched[2] = {0, 0};
+        if (MODE == R8_DQ && chunk > 0) {
+            const char* qb = reinterpret_cast<const char*>(a.Qrow) + (hoff * D + (size_t)dh * (D / 2)) * sizeof(T);
+            constexpr int LINES = (D / 2) * (int)sizeof(T) / 128;   // 128-byte lines of this wave's half of a row
+#pragma unroll
+            for (int r = 0; r < 2; r++) {
+#pragma unroll
+                for (int ln = 0; ln < LINES; ln += 2) {
+                    if (ln + h < LINES)   // (the two lanes of a row take a line each; never past the end of the half row)
+                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * D * sizeof(T) + 128 * (ln + h));
+                }
+            }
+        }
+        if (MODE == R8_DQ && chunk == 0) {
             // Per-row scalars of the backward for row block r = dh of the row group (the producers need them from their
             // first tile on, the column kernel reads them from global memory): this role idles until the first P arrives.
+            // (Behind the first chunk the producers compute them: see there.)
             const T* X = reinterpret_cast<const T*>(a.X) + hoff * D;
             const int rc = rowc[dh];
             frag xs[NS];
@@ -520,6 +555,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                     }
             }
             if constexpr (MODE == R8_DQ) {
+                asm volatile("" ::"v"(touched[0]), "v"(touched[1]));
                 // Row sums of dD over the keys before the chunk: q_i . dQ_i of what the accumulators hold now; this wave's
                 // half of the columns goes to LDS, the halves meet behind the next barrier
                 const T* Qh = reinterpret_cast<const T*>(a.Qrow) + hoff * D + (size_t)dh * (D / 2);
