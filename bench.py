@@ -2,13 +2,17 @@
 """Headline benchmark: mLSTM matmul-form forward + backward, B4 H8 S4096 D256 bf16 (fp32 accumulation), one MI355X.
 
 One step = one forward (h, m, b) plus one backward (dq, dk, dv, df, di) through the C ABI of libmlstm_hip.so, inputs
-resident in HBM.  Prints ONE JSON line.  `value` is algorithmic TFLOP/s: 7*D*S*(S+1) useful (causal) multiply-add
-flops per head and step (2 products forward, 5 backward) divided by wall time; tokens/s is reported beside it.
-`roofline` is the dominant kernel (the column-parallel backward tile kernel) timed with HIP events on its launch
-stream during the timed steps; `cpu_baseline` times the C restatement of the reference's CPU path on one head.
+resident in HBM (the same buffers every step: 256 MiB of them, which the chip's 256 MB last-level cache may keep).
+Prints ONE JSON line.  `value` is algorithmic TFLOP/s: 7*D*S*(S+1) useful (causal) multiply-add flops per head and step
+(2 products forward, 5 backward) divided by wall time; long 16-bit sequences run in chunks and execute far fewer flops
+than that, which `executed_tflops` / `executed_frac` report beside it.  `roofline` is the dominant kernel (the
+column-parallel backward tile kernel) timed with HIP events on its launch stream during the timed steps;
+`cpu_baseline` times the C restatement of the reference's CPU path, `cpu_baseline_torch` the dense PyTorch formulas, on
+the same seeded inputs; `secondary` holds the other workloads (long context, scan form, split mode), each measured the
+same way with a roofline object of its own.
 """
 import argparse
-import ctypes
+import hashlib
 import json
 import os
 import sys
@@ -28,27 +32,62 @@ WORKLOADS = {
     "aux_B4_H8_S4096_D256_f16": (4, 8, 4096, 256, torch.float16, 3.0, 0.0, 1.0),
 }
 PEAK_TFLOPS = {torch.bfloat16: 2500.0, torch.float16: 2500.0, torch.float32: 157.3}
-# HBM bytes per launch of the column kernel (in chunks of 512, the default at this shape), from two `rocprofv3 --pmc`
-# runs of this script with --calibrate-copy (FETCH_SIZE 172673, WRITE_SIZE 142080 per dispatch; the 256 MiB copy in the
-# same runs reads 131096 / 262144, so the fetch counter is scaled by 2.0 and the write counter by 1.0; both are then KiB).
-COL_KERNEL_HBM_BYTES = {"cfg4_B4_H8_S4096_D256_bf16": (2.0 * 172673 + 1.0 * 142080) * 1024}
 DTYPE_NAME = {torch.bfloat16: "bf16", torch.float16: "f16", torch.float32: "f32"}
+CSRC = os.path.join(ROOT, "xlstm-triton-cuda-implementation_amd", "csrc")
 
 
-def cpu_baseline(S, D, f_mean, heads=3):
-    """`heads` of the workload's heads through the C oracle (dense S x S, fp32, single thread like the reference's
-    cpu_utils.cuh): about 4.4 s per head at S=4096, D=256 on the GPU box's host.  Returns the JSON object."""
-    import numpy as np
+def kernel_source_hash():
+    """Identifies the kernels a measured traffic figure belongs to: sha256 over the device sources."""
+    hsh = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".hip", ".h")):
+            hsh.update(name.encode())
+            hsh.update(open(os.path.join(CSRC, name), "rb").read())
+    return hsh.hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel, chunk):
+    """HBM bytes per launch of `kernel` from profiles/traffic.json (two rocprofv3 --pmc runs, see the file), or None when the
+    figure on file was taken with other kernel sources or another chunk length."""
+    try:
+        table = json.load(open(os.path.join(ROOT, "profiles", "traffic.json")))
+    except (OSError, ValueError):
+        return None
+    rec = table.get(workload, {}).get(kernel)
+    if not rec or rec.get("source_hash") != kernel_source_hash() or rec.get("chunk_len") != chunk:
+        return None
+    return float(rec["hbm_bytes_per_launch"])
+
+
+def make_inputs(B, NH, S, D, dtype, f_mean, i_mean, dh_std, with_o=False, seed=0):
+    """The seeded recipe shared by the tests, the CPU baselines and this benchmark: one CPU generator, fp32 normal draws in
+    the order q, k, v, f, i, dh (, o), affine transform, cast to the workload's type."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, NH, S, D), generator=g)
+    k = torch.randn((B, NH, S, D), generator=g)
+    v = torch.randn((B, NH, S, D), generator=g)
+    f = torch.randn((B, NH, S), generator=g) + f_mean
+    i = torch.randn((B, NH, S), generator=g) + i_mean
+    dh = torch.randn((B, NH, S, D), generator=g) * dh_std
+    out = [q, k, v, f, i, dh]
+    if with_o:
+        out.append(torch.randn((B, NH, S, D), generator=g))
+    return [x.to(dtype) for x in out]
+
+
+def cpu_baseline(host, S, D, heads=3):
+    """`heads` of the workload's heads (its own seeded inputs, upcast to fp32) through the C oracle: dense S x S, fp32,
+    single thread like the reference's cpu_utils.cuh; about 4.4 s per head at S=4096, D=256 on the GPU box's host."""
     from oracle import c_oracle as C
+    q, k, v, f, i, dh = host
+    NH = q.shape[1]
     dt = 0.0
     for head in range(heads):
-        rng = np.random.default_rng(head)
-        q, k, v, dh = (rng.standard_normal((S, D)).astype(np.float32) for _ in range(4))
-        f = (rng.standard_normal(S) + f_mean).astype(np.float32)
-        i = rng.standard_normal(S).astype(np.float32)
+        bi, hi = divmod(head, NH)
+        a = [x[bi, hi].float().numpy().copy() for x in (q, k, v, f, i, dh)]
         t0 = time.perf_counter()
-        C.forward_f32(q, k, v, f, i, threads=1)
-        C.backward_f32(dh, q, k, v, f, i, threads=1)
+        C.forward_f32(a[0], a[1], a[2], a[3], a[4], threads=1)
+        C.backward_f32(a[5], a[0], a[1], a[2], a[3], a[4], threads=1)
         dt += time.perf_counter() - t0
     flops = heads * 7.0 * D * S * (S + 1)
     return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
@@ -56,15 +95,144 @@ def cpu_baseline(S, D, f_mean, heads=3):
             "tokens_per_s": heads * S / dt}
 
 
-def bench_scan(args, ffi):
-    """Secondary workload: scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape)."""
+def cpu_baseline_torch(host, S, D, heads=2):
+    """The dense PyTorch formulas of the reference (mlstm_matmul.py:104-118, :336-365, restated in oracle/mlstm_oracle.py)
+    in fp32 on `heads` heads with torch's intra-op threads."""
+    from oracle import mlstm_oracle as O
+    q, k, v, f, i, dh = host
+    NH = q.shape[1]
+    dt = 0.0
+    for head in range(heads):
+        bi, hi = divmod(head, NH)
+        a = [x[bi:bi + 1, hi:hi + 1] for x in (q, k, v, f, i, dh)]
+        t0 = time.perf_counter()
+        O.mlstm_forward_dense(*a[:5], dtype=torch.float32)
+        O.mlstm_backward_dense(a[5], *a[:5], dtype=torch.float32)
+        dt += time.perf_counter() - t0
+    flops = heads * 7.0 * D * S * (S + 1)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"{heads} of the workload's heads (S={S}, D={D}), forward+backward, dense torch fp32 formulas, {dt:.1f} s",
+            "tokens_per_s": heads * S / dt}
+
+
+def chunk_work(S, D, BH, chunk, el):
+    """Flops the kernels execute per step in chunks of `chunk`, and the column kernel's share, with its compulsory bytes."""
+    lens = [min(chunk, S - c0) for c0 in range(0, S, chunk)]
+    pair_unit = float(D) * sum(n * (n + 1) for n in lens) * BH            # one product over the (query, key) pairs inside chunks
+    state_rows = float(sum(lens[1:])) * BH                                 # positions that read a forward state
+    state_keys = float(sum(lens[:-1])) * BH                                # positions that read a reverse state
+    sums = 2.0 * D * D * (sum(lens[:-1]) + sum(lens[1:])) * BH             # chunk sums, both directions (2 D^2 per position)
+    executed = 8.0 * pair_unit + 2.0 * D * D * 2 * state_rows + 2.0 * D * D * 2 * state_keys + sums
+    col_flops = 4.0 * pair_unit + 2.0 * D * D * 2 * state_keys            # four products per pair, two with the reverse state
+    tiles_met = sum((n // 64 + 1) / 2.0 * n for n in lens)
+    col_bytes = BH * (S * D * el * 6 + tiles_met * 4 + (len(lens) - 1) * (D * D * el + 4.0 * D))
+    return executed, col_flops, col_bytes
+
+
+def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
+    """Times `steps` forward + backward steps of one matmul-form workload.  Returns (json object, host inputs)."""
+    L = ffi.lib()
+    B, NH, S, D, dtype, f_mean, i_mean, dh_std = WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    if host is None:
+        host = make_inputs(B, NH, S, D, dtype, f_mean, i_mean, dh_std)
+    q, k, v, f, i, dh = (x.to(dev) for x in host)
+    h, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
+    m, b = (torch.empty((B, NH, S), device=dev, dtype=torch.float32) for _ in range(2))
+    df, di = torch.empty_like(f), torch.empty_like(i)
+    dt_code, gate_code = ffi.dtype_code(dtype, precise), ffi.dtype_code(dtype)
+    ws, ws_n = ffi.workspace(ffi.OP_BACKWARD, B, NH, S, D, dt_code, dev)
+    st, P = ffi.stream_ptr(), ffi.ptr
+    # what Triton_mLSTM.apply(...).backward(dh) runs: the forward keeps (h, m, b) and what its backward can reuse
+    nsaved = int(L.mlstm_saved_state_bytes(B, NH, S, D, dt_code))
+    saved = torch.empty(max(nsaved, 1), dtype=torch.uint8, device=dev)
+
+    def step():
+        rc = L.mlstm_forward_save_ex(P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, B, NH, S, D, dt_code, gate_code,
+                                     P(ws), ws_n, st)
+        ffi.check_rc(rc, "mlstm_forward_save_ex")
+        rc = L.mlstm_backward_saved_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, P(dq), P(dk), P(dv),
+                                       P(df), P(di), B, NH, S, D, dt_code, gate_code, P(ws), ws_n, st)
+        ffi.check_rc(rc, "mlstm_backward_saved_ex")
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    # HIP events inside the timed region bracket the dominant kernel only, on every fourth step: an event pair holds
+    # the stream idle for about 10 us, and with all six kernel groups timed on every step that was 9 % of the step
+    ffi.timing_select(["col"], every=4)
+    ffi.timing_enable(True)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    kern = {"col": ffi.timing_read("col")}
+    # the other kernels' durations, for the breakdown: a few more steps, outside the timed region, all kernels timed
+    ffi.timing_select(None, every=1)
+    for _ in range(max(steps // 4, 1)):
+        step()
+    torch.cuda.synchronize()
+    ffi.timing_enable(False)
+    for kname in ("gates", "chunk_states", "row_fwd", "row_dq", "df"):
+        kern[kname] = ffi.timing_read(kname)
+    ffi.timing_read("col")
+    kern = {kname: kern[kname] for kname in ("gates", "chunk_states", "row_fwd", "col", "row_dq", "df")}
+    assert L.mlstm_kernel_error() == 0, "a kernel's bounded wait expired during the benchmark"
+
+    ms_step = (t1 - t0) * 1e3 / steps
+    BH = B * NH
+    unit_flops = float(D) * S * (S + 1) * BH            # one causal product over the whole batch
+    tflops = 7.0 * unit_flops / (ms_step * 1e-3) / 1e12
+    peak = PEAK_TFLOPS[dtype]
+    col_ms = kern["col"][0] / max(kern["col"][1], 1)
+    chunk = int(L.mlstm_chunk_length_for(S, D, dt_code))
+    el = torch.empty(0, dtype=dtype).element_size()
+    if chunk > 0 and (S + 63) // 64 <= 1024:
+        executed, col_flops, col_bytes = chunk_work(S, D, BH, chunk, el)
+    else:
+        # every key tile: 8 products executed (dH V^T in both backward kernels), 4 of them in the column kernel; the split
+        # mode runs each of the 4 second products (P V, G K, G^T Q, W^T dH) a second time on the low-order terms
+        chunk = 0
+        executed = (12.0 if precise else 8.0) * unit_flops
+        col_flops = (6.0 if precise else 4.0) * unit_flops
+        col_bytes = BH * (S * D * el * 6 + (S / 64 + 1) / 2.0 * S * 4)
+    achieved = col_flops / (col_ms * 1e-3) / 1e12 if col_ms > 0 else 0.0
+    hbm_achieved = col_bytes / (col_ms * 1e-3) / 1e9 if col_ms > 0 else 0.0
+    col_kernel = "col_kernel" if (precise or dtype == torch.float32 or D == 64) else "col16_kernel"
+    traffic = measured_traffic(name + ("+precise" if precise else ""), col_kernel, chunk)
+    out = {
+        "metric": "mLSTM matmul-form fwd+bwd algorithmic TFLOP/s (7*D*S*(S+1) per head), " + name + (" split mode" if precise else ""),
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": DTYPE_NAME[dtype], "data": "synthetic",
+        "config": {"workload": name, "B": B, "NH": NH, "S": S, "D": D, "f": f"N({f_mean},1)", "i": f"N({i_mean},1)",
+                   "chunk_len": chunk, "split_mode": bool(precise)},
+        "tokens_per_s": B * S / (ms_step * 1e-3),
+        "algorithmic_frac": tflops / peak,
+        "executed_tflops": executed / (ms_step * 1e-3) / 1e12,
+        "executed_frac": executed / (ms_step * 1e-3) / 1e12 / peak,
+        "kernel_ms": {n: (t / c if c else None) for n, (t, c) in kern.items()},
+    }
+    mfma = {"mfma_tflops": achieved, "mfma_frac": achieved / peak}
+    hbm = {"hbm_gbs": hbm_achieved, "hbm_frac": hbm_achieved / 8000.0}
+    if achieved / peak >= hbm_achieved / 8000.0:
+        out["roofline"] = {"bound": "mfma", "kernel": col_kernel + " (dK, dV, dI)", "achieved": achieved, "peak": peak,
+                           "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic, **hbm}
+    else:
+        # in chunks a workgroup meets few query tiles and the kernel is nearer to the HBM roof than to the MFMA roof
+        out["roofline"] = {"bound": "hbm", "kernel": col_kernel + " (dK, dV, dI), chunks of %d" % chunk, "achieved": hbm_achieved,
+                           "peak": 8000.0, "unit": "GB/s", "frac": hbm_achieved / 8000.0, "traffic": traffic, **mfma}
+    return out, host
+
+
+def run_scan(ffi, steps, warmup):
+    """Scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape)."""
     L = ffi.lib()
     B, NH, S, D = 1, 4, 2048, 1024
     dev = torch.device("cuda:0")
-    g = torch.Generator(device=dev).manual_seed(0)
-    mk = lambda *s: torch.randn(s, generator=g, device=dev, dtype=torch.float32)
-    q, k, v, o = (mk(B, NH, S, D) for _ in range(4))
-    f, i = mk(B, NH, S), mk(B, NH, S)
+    host = make_inputs(B, NH, S, D, torch.float32, 0.0, 0.0, 1.0, with_o=True)
+    q, k, v, f, i, _, o = (x.to(dev) for x in host)
     h = torch.empty_like(q)
     ws, ws_n = ffi.workspace(ffi.OP_SCAN_FORWARD, B, NH, S, D, ffi.F32, dev)
     st, P = ffi.stream_ptr(), ffi.ptr
@@ -73,36 +241,41 @@ def bench_scan(args, ffi):
         ffi.check_rc(L.mlstm_scan_forward_ex(P(q), P(k), P(v), P(f), P(i), P(o), P(h), B, NH, S, D, ffi.F32, P(ws), ws_n, st),
                      "mlstm_scan_forward_ex")
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    ffi.timing_enable(True)
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    ffi.timing_select(None, every=1)
+    ffi.timing_enable(True)
+    for _ in range(max(steps // 4, 1)):
+        step()
+    torch.cuda.synchronize()
     ffi.timing_enable(False)
     kern = {name: ffi.timing_read(name) for name in ("gates", "scan_carry", "scan_state", "scan_out")}
-    ms_step = (t1 - t0) * 1e3 / args.steps
+    ms_step = (t1 - t0) * 1e3 / steps
     BH = B * NH
     bytes_compulsory = (5.0 * BH * S * D + 3.0 * BH * S) * 4          # q, k, v, o in, h out, f, i in (+ m)
     flops = BH * (S / 64.0) * (2 * 64 * D * D * 2 + 2 * 2 * D * 64 * 65 / 2 * 2)  # state update + read-out, in-chunk pairs
     st_ms = kern["scan_state"][0] / max(kern["scan_state"][1], 1)
-    out = {
+    t_fl = flops / (st_ms * 1e-3) / 1e12 if st_ms else 0.0
+    return {
         "metric": "mLSTM scan-form forward, compulsory HBM GB/s, cfg3_B1_H4_S2048_D1024_f32",
-        "value": bytes_compulsory / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": bytes_compulsory / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "cfg3_B1_H4_S2048_D1024_f32", "B": B, "NH": NH, "S": S, "D": D},
         "tokens_per_s": B * S / (ms_step * 1e-3), "fp32_tflops": flops / (ms_step * 1e-3) / 1e12,
         "kernel_ms": {n: (t / c if c else None) for n, (t, c) in kern.items()},
-        "roofline": {"bound": "mfma", "kernel": "scan_intra_kernel + scan_state_kernel (fp32 MFMA)",
-                     "achieved": flops / (st_ms * 1e-3) / 1e12 if st_ms else 0.0, "peak": 157.3, "unit": "TFLOP/s",
-                     "frac": (flops / (st_ms * 1e-3) / 1e12 / 157.3) if st_ms else 0.0, "traffic": None},
-        "hbm_frac_compulsory": bytes_compulsory / (ms_step * 1e-3) / 8e12,
+        # the binding roof: 38.7 GF of fp32 matrix work against 168 MB of compulsory traffic (ridge at 20 flop/B, the
+        # workload has 230); both fractions are reported
+        "roofline": {"bound": "mfma", "kernel": "scan_state_kernel (fp32 MFMA)", "achieved": t_fl, "peak": 157.3, "unit": "TFLOP/s",
+                     "frac": t_fl / 157.3, "traffic": measured_traffic("cfg3_B1_H4_S2048_D1024_f32", "scan_state_kernel", 64),
+                     "hbm_gbs": bytes_compulsory / (ms_step * 1e-3) / 1e9, "hbm_frac": bytes_compulsory / (ms_step * 1e-3) / 8e12},
     }
-    print(json.dumps(out))
 
 
 def main():
@@ -112,6 +285,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (torch) before the steps: under rocprofv3 --pmc its "
@@ -126,120 +300,26 @@ def main():
 
     from _mlstm_pkg import submodule
     ffi = submodule("_ffi")
-    if args.workload == "cfg3_scan":
-        return bench_scan(args, ffi)
-    L = ffi.lib()
-    B, NH, S, D, dtype, f_mean, i_mean, dh_std = WORKLOADS[args.workload]
-    dev = torch.device("cuda:0")
-    g = torch.Generator(device=dev).manual_seed(0)
-    mk = lambda *s: torch.randn(s, generator=g, device=dev, dtype=torch.float32)
-    q, k, v = (mk(B, NH, S, D).to(dtype) for _ in range(3))
-    f = (mk(B, NH, S) + f_mean).to(dtype)
-    i = (mk(B, NH, S) + i_mean).to(dtype)
-    dh = (mk(B, NH, S, D) * dh_std).to(dtype)
-    h, dq, dk, dv = (torch.empty_like(q) for _ in range(4))
-    m, b = (torch.empty((B, NH, S), device=dev, dtype=torch.float32) for _ in range(2))
-    df, di = torch.empty_like(f), torch.empty_like(i)
-    dt_code = ffi.dtype_code(dtype, args.precise)
-    gate_code = ffi.dtype_code(dtype)
-    ws, ws_n = ffi.workspace(ffi.OP_BACKWARD, B, NH, S, D, dt_code, dev)
-    st = ffi.stream_ptr()
-    P = ffi.ptr
-
-    # what Triton_mLSTM.apply(...).backward(dh) runs: the forward keeps (h, m, b) and, for sequences that run in chunks,
-    # the states at the chunk ends for its backward
-    nsaved = int(L.mlstm_saved_state_bytes(B, NH, S, D, dt_code))
-    saved = torch.empty(max(nsaved, 1), dtype=torch.uint8, device=dev)
-
-    def step():
-        rc = L.mlstm_forward_save_ex(P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, B, NH, S, D, dt_code, gate_code,
-                                     P(ws), ws_n, st)
-        ffi.check_rc(rc, "mlstm_forward_save_ex")
-        rc = L.mlstm_backward_saved_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(h), P(m), P(b), P(saved), nsaved, P(dq), P(dk), P(dv),
-                                       P(df), P(di), B, NH, S, D, dt_code, gate_code, P(ws), ws_n, st)
-        ffi.check_rc(rc, "mlstm_backward_saved_ex")
-
     if args.calibrate_copy:
-        src = torch.ones(64 * 1024 * 1024, device=dev, dtype=torch.float32)
+        src = torch.ones(64 * 1024 * 1024, device="cuda:0", dtype=torch.float32)
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # HIP events inside the timed region bracket the dominant kernel only, on every fourth step: an event pair holds
-    # the stream idle for about 10 us, and with all six kernel groups timed on every step that was 9 % of the step
-    ffi.timing_select(["col"], every=4)
-    ffi.timing_enable(True)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    kern = {"col": ffi.timing_read("col")}
-    # the other kernels' durations, for the breakdown: a few more steps, outside the timed region, all kernels timed
-    ffi.timing_select(None, every=1)
-    for _ in range(max(args.steps // 4, 1)):
-        step()
-    torch.cuda.synchronize()
-    ffi.timing_enable(False)
-    for name in ("gates", "chunk_states", "row_fwd", "row_dq", "df"):
-        kern[name] = ffi.timing_read(name)
-    ffi.timing_read("col")
-    kern = {name: kern[name] for name in ("gates", "chunk_states", "row_fwd", "col", "row_dq", "df")}
-
-    ms_step = (t1 - t0) * 1e3 / args.steps
-    BH = B * NH
-    unit_flops = float(D) * S * (S + 1) * BH            # one causal product over the whole batch
-    flops_step = 7.0 * unit_flops
-    tflops = flops_step / (ms_step * 1e-3) / 1e12
-    tokens_s = B * S / (ms_step * 1e-3)
-
-    # dominant kernel: column-parallel backward tile kernel, 3 of the 7 algorithmic products (QK^T recompute, dK, dV);
-    # the fourth product it executes (dH V^T) is counted once, in the dQ kernel's share.  In chunks it only meets the
-    # (query, key) pairs inside a chunk and its algorithmic work is counted over those pairs, sum over the chunks of
-    # D * len * (len + 1) per product and head, plus the two products keys x reverse state (2 D^2 per key and product)
-    # that bring in the queries behind the chunk.
-    col_ms = kern["col"][0] / max(kern["col"][1], 1)
-    chunk = int(L.mlstm_chunk_length_for(S, D, dt_code))
-    el = torch.empty(0, dtype=dtype).element_size()
-    if chunk > 0 and (S + 63) // 64 <= 1024:
-        lens = [min(chunk, S - c0) for c0 in range(0, S, chunk)]
-        col_unit = float(D) * sum(n * (n + 1) for n in lens) * BH
-        state_flops = 2.0 * 2.0 * D * D * sum(lens[:-1]) * BH
-        state_bytes = (len(lens) - 1) * (2.0 * D * D * el + 4.0 * D)
-    else:
-        chunk, col_unit, state_flops, state_bytes = 0, unit_flops, 0.0, 0.0
-    col_flops = 3.0 * col_unit + state_flops
-    peak = PEAK_TFLOPS[dtype]
-    achieved = col_flops / (col_ms * 1e-3) / 1e12 if col_ms > 0 else 0.0
-    # its compulsory HBM bytes: Q, dH, K, V once; dK, dV written; the row partials of the key tiles a position meets;
-    # in chunks the reverse states in both layouts and their vectors
-    tiles_met = sum((min(chunk, S - c0) // 64 + 1) / 2.0 * min(chunk, S - c0) for c0 in range(0, S, chunk)) if chunk else (S / 64 + 1) / 2.0 * S
-    col_bytes = BH * (S * D * el * 6 + tiles_met * 4 + state_bytes)
-    hbm_achieved = col_bytes / (col_ms * 1e-3) / 1e9 if col_ms > 0 else 0.0
-    out = {
-        "metric": "mLSTM matmul-form fwd+bwd algorithmic TFLOP/s (7*D*S*(S+1) per head), " + args.workload,
-        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": DTYPE_NAME[dtype], "data": "synthetic",
-        "config": {"workload": args.workload, "B": B, "NH": NH, "S": S, "D": D, "f": f"N({f_mean},1)", "i": f"N({i_mean},1)"},
-        "tokens_per_s": tokens_s,
-        "frac_of_peak": tflops / peak,
-        "kernel_ms": {n: (t / c if c else None) for n, (t, c) in kern.items()},
-    }
-    traffic = COL_KERNEL_HBM_BYTES.get(args.workload) if chunk == 512 or not chunk else None
-    if achieved / peak >= hbm_achieved / 8000.0:
-        out["roofline"] = {"bound": "mfma", "kernel": "col16_kernel (dK, dV, dI)", "achieved": achieved, "peak": peak,
-                           "unit": "TFLOP/s", "frac": achieved / peak, "traffic": traffic}
-    else:
-        # in chunks a workgroup meets few query tiles and the kernel is nearer to the HBM roof than to the MFMA roof
-        out["roofline"] = {"bound": "hbm", "kernel": "col16_kernel (dK, dV, dI), chunks of %d" % chunk, "achieved": hbm_achieved,
-                           "peak": 8000.0, "unit": "GB/s", "frac": hbm_achieved / 8000.0, "traffic": traffic,
-                           "mfma_tflops": achieved, "mfma_frac": achieved / peak}
+    if args.workload == "cfg3_scan":
+        print(json.dumps(run_scan(ffi, args.steps, args.warmup)))
+        return
+    out, host = run_matmul(ffi, args.workload, args.steps, args.warmup, precise=args.precise)
+    headline = args.workload == "cfg4_B4_H8_S4096_D256_bf16" and not args.precise
+    if headline and not args.no_secondary:
+        few = max(min(args.steps, 20), 5)
+        out["secondary"] = [run_matmul(ffi, args.workload, few, 3, precise=True, host=host)[0],
+                            run_matmul(ffi, "cfg5_B2_H32_S16384_D128_bf16", few, 3)[0],
+                            run_scan(ffi, max(args.steps, 20), 5)]
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(S, D, f_mean)
+        S, D = WORKLOADS[args.workload][2:4]
+        out["cpu_baseline"] = cpu_baseline(host, S, D)
+        out["cpu_baseline_torch"] = cpu_baseline_torch(host, S, D)
     print(json.dumps(out))
 
 
