@@ -117,7 +117,14 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
     const int jlast = wave_active ? r0 / GRAN : -1;
     const int jfull = wave_active ? r0 / GRAN : 0;
 
-    for (int g = tid; g < NG; g += 512) sG[g] = a.G2[goff + g];
+    // Every trip to memory in this prologue costs thousands of cycles, so the independent ones are requested back to back
+    // and their values used as late as possible: the granule bases are asked for here and stored to LDS just before the
+    // first barrier.
+    const double g_mine = tid < NG ? a.G2[goff + tid] : 0.0;
+    auto store_granule_bases = [&]() {
+        if (tid < NG) sG[tid] = g_mine;
+        for (int g = tid + 512; g < NG; g += 512) sG[g] = a.G2[goff + g];
+    };
     if (tid < 2) pcnt[tid] = 0;
 
     TileDma<T, D, GRAN, 256> tdma;
@@ -273,33 +280,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             p_rg[(4 + 2 * kh + 1) * 64] = f11;
         };
 
-        if constexpr (MODE == R8_FWD) {
-            if (chunk > 0) {
-                // Row sums: what lies before the chunk contributes decay_i (q_i . n~) with the vector state n~ of the
-                // previous chunk; the two producers of a row group take half of the contraction each.  The consumers
-                // meanwhile add decay_i q_i^T C~ to their accumulators (state tiles through the Y2 stages, two per round).
-                const float* nst = a.Nst + ((size_t)bh * a.n_states + chunk - 1) * D + 8 * h;
-                float part[2] = {0.f, 0.f};
-                auto half_dot = [&](auto first_tag) {   // (the fragment index must be a constant: xf lives in registers)
-                    constexpr int S0 = decltype(first_tag)::value;
-#pragma unroll
-                    for (int s = S0; s < S0 + NS / 2; s++) {
-                        const f32x4 n0 = *reinterpret_cast<const f32x4*>(nst + KW * s), n1 = *reinterpret_cast<const f32x4*>(nst + KW * s + 4);
-#pragma unroll
-                        for (int r = 0; r < 2; r++) {
-                            const f32x8 qv = __builtin_convertvector(xf[r][s], f32x8);
-#pragma unroll
-                            for (int e = 0; e < 4; e++) part[r] += qv[e] * n0[e] + qv[4 + e] * n1[e];
-                        }
-                    }
-                };
-                if (kh == 0) half_dot(std::integral_constant<int, 0>{});
-                else half_dot(std::integral_constant<int, NS / 2>{});
-#pragma unroll
-                for (int r = 0; r < 2; r++)
-                    bsum[r] = part[r] * fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
-            }
-        }
+        store_granule_bases();
         __syncthreads();  // sG, counters visible; plain global loads above are done (pin)
         if constexpr (MODE == R8_DQ) {   // 1/n and db of the wave's rows, computed by the consumers while this role loaded its rows
 #pragma unroll
@@ -363,6 +344,34 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 for (int x = 0; x < 16; x++) { s0[x] = 0.f; s1[x] = 0.f; }
             }
             publish(s0, s1, j);
+        }
+        if constexpr (MODE == R8_FWD) {
+            if (chunk > 0) {
+                // Row sums: what lies before the chunk contributes decay_i (q_i . n~) with the vector state n~ of the
+                // previous chunk; the two producers of a row group take half of the contraction each.  Done here, behind
+                // the tile loop, where this role has time to spare (the consumers are one tile behind): in the prologue
+                // the loads of n~ were one more trip to memory on the workgroup's critical path.
+                const float* nst = a.Nst + ((size_t)bh * a.n_states + chunk - 1) * D + 8 * h;
+                float part[2] = {0.f, 0.f};
+                auto half_dot = [&](auto first_tag) {   // (the fragment index must be a constant: xf lives in registers)
+                    constexpr int S0 = decltype(first_tag)::value;
+#pragma unroll
+                    for (int s = S0; s < S0 + NS / 2; s++) {
+                        const f32x4 n0 = *reinterpret_cast<const f32x4*>(nst + KW * s), n1 = *reinterpret_cast<const f32x4*>(nst + KW * s + 4);
+#pragma unroll
+                        for (int r = 0; r < 2; r++) {
+                            const f32x8 qv = __builtin_convertvector(xf[r][s], f32x8);
+#pragma unroll
+                            for (int e = 0; e < 4; e++) part[r] += qv[e] * n0[e] + qv[4 + e] * n1[e];
+                        }
+                    }
+                };
+                if (kh == 0) half_dot(std::integral_constant<int, 0>{});
+                else half_dot(std::integral_constant<int, NS / 2>{});
+#pragma unroll
+                for (int r = 0; r < 2; r++)
+                    bsum[r] += part[r] * fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
+            }
         }
         dma_wait();
         // Output gate: this wave is done while the consumer of the same rows still has its last product and the
@@ -504,6 +513,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
             }
         }
+        store_granule_bases();
         __syncthreads();
         if (chunk > 0) {
             // What lies before the chunk: the state at the end of the previous chunk, D rows of D entries, as D/64 tiles
