@@ -50,6 +50,7 @@ extern "C" {
 #define MLSTM_OP_SCAN_FORWARD 2
 #define MLSTM_OP_FORWARD_GATED 3
 #define MLSTM_OP_BACKWARD_GATED 4
+#define MLSTM_OP_SCAN_BACKWARD 5
 
 /*
  * Single-head fp16 forward, D = 128, default stream: the launch of the CUDA harness,
@@ -155,6 +156,18 @@ int mlstm_scan_forward_ex(const void* q, const void* k, const void* v, const voi
                           void* h, int B, int NH, int S, int D, int dtype, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/*
+ * Backward of mlstm_scan(): gradients of q, k, v, f, i, o from the gradient of the gated output.  The reference has
+ * no kernel for it (mlstm_scan.py holds a forward only; its differentiable counterpart is the PyTorch
+ * mlstm_scan_pytorch, mlstm_scan.py:343-380); the gradients are those of mlstm_matmul.py:150-333 behind the gate of
+ * mlstm_scan.py:277, evaluated with the scan form's own kernels (causal weighted sums with a matrix state carried
+ * over chunks of 64 positions), so every head dimension of the forward is served.  Recomputes the forward: only the
+ * inputs are needed.  fp32 only; dF[..., 0] = 0.  Workspace: mlstm_workspace_bytes(MLSTM_OP_SCAN_BACKWARD, ...).
+ */
+int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
+                           const void* o, void* dq, void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S,
+                           int D, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+
 /* Bytes of scratch the operation needs for this shape (the torch.zeros workspaces of mlstm_scan.py:299-307 and
  * the db buffer of mlstm_matmul.py:394 are the reference's counterparts). */
 size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype);
@@ -175,6 +188,7 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype);
 #define MLSTM_K_SCAN_OUT 8
 #define MLSTM_K_GATE_BWD 9  /* element-wise backward of the output gate (gated matmul form only) */
 #define MLSTM_K_CHUNK_STATES 10  /* chunk sums + carry of the chunked forward (16-bit, D = 128 / 256, long sequences) */
+#define MLSTM_K_SCAN_GLUE 11     /* row-wise and vector-sum kernels between the scans of the scan form's backward */
 int mlstm_timing_enable(int on);
 /* An event pair costs the stream about 10 us of idle time around the launch it brackets.  mlstm_timing_select narrows
  * the timing to the kernels whose bit (1u << MLSTM_K_...) is set in `mask` and, of their launches, to every

@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(_HERE, "libmlstm_hip.so")
 
 F32, F16, BF16 = 0, 1, 2
 PRECISE = 0x100   # MLSTM_PRECISE, or-ed into the dtype code: split mode of the 16-bit kernels
-OP_FORWARD, OP_BACKWARD, OP_SCAN_FORWARD, OP_FORWARD_GATED, OP_BACKWARD_GATED = 0, 1, 2, 3, 4
+OP_FORWARD, OP_BACKWARD, OP_SCAN_FORWARD, OP_FORWARD_GATED, OP_BACKWARD_GATED, OP_SCAN_BACKWARD = 0, 1, 2, 3, 4, 5
 NOALLOC_MAX_WORKSPACE = 8 << 20   # MLSTM_NOALLOC_MAX_WORKSPACE
 _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dtype)",
@@ -55,6 +55,8 @@ def lib():
         L.mlstm_backward_gated_ex.argtypes = [vp] * 16 + [ci] * 6 + [vp, sz, vp]
         L.mlstm_scan_forward_ex.restype = ci
         L.mlstm_scan_forward_ex.argtypes = [vp] * 7 + [ci] * 5 + [vp, sz, vp]
+        L.mlstm_scan_backward_ex.restype = ci
+        L.mlstm_scan_backward_ex.argtypes = [vp] * 13 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_timing_enable.restype = ci
         L.mlstm_timing_enable.argtypes = [ci]
         L.mlstm_timing_select.restype = ci
@@ -77,6 +79,7 @@ def lib():
 
 def exported_symbols():
     return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
+            "mlstm_scan_backward_ex",
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
@@ -84,7 +87,7 @@ def exported_symbols():
 
 
 KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
-           "scan_out": 8, "gate_bwd": 9, "chunk_states": 10}
+           "scan_out": 8, "gate_bwd": 9, "chunk_states": 10, "scan_glue": 11}
 
 
 def force_generic_kernels(on):

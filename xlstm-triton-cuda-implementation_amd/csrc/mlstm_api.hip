@@ -337,6 +337,8 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype) {
         case MLSTM_OP_SCAN_FORWARD:  // gates, m, row sums, in-chunk pairs, vector states, partial numerators
             return z.fwd() + up256(z.BH * z.NG * 64 * 64 * 4) + up256(z.BH * z.NG * z.D * 4) +
                    (size_t)(scan_key_splits((int)z.BH, D) - 1) * up256(z.BH * z.S * z.D * 4);
+        case MLSTM_OP_SCAN_BACKWARD:
+            return (D % 64 == 0 && D >= 64) ? scan_backward_workspace_bytes((int)z.BH, S, D) : 0;
     }
     return 0;
 }
@@ -623,6 +625,25 @@ int mlstm_scan_forward_ex(const void* q, const void* k, const void* v, const voi
     a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.P = P; a.Nst = Nst; a.hpart = hpart;
     a.BH = (int)z.BH; a.S = (int)z.S; a.D = D; a.NC = (int)z.NG;
     return launch_scan(a, KS, st, scan_mark);
+}
+
+int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
+                           const void* o, void* dq, void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S, int D,
+                           int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!dh_gated || !q || !k || !v || !f || !i || !o || !dq || !dk || !dv || !df || !di || !d_o || B <= 0 || NH <= 0 || S <= 0)
+        return MLSTM_EINVAL;
+    if (dtype != MLSTM_F32) return MLSTM_ESHAPE;
+    if (!(D == 64 || D == 128 || D == 256 || D == 512 || D == 1024) || S > 131072) return MLSTM_ESHAPE;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const size_t need = scan_backward_workspace_bytes(B * NH, S, D);
+    Scratch sc;
+    if (int rc = sc.get(workspace, workspace_bytes, need, st)) return rc;
+    ScanBwdArgs a{};
+    a.dhg = (const float*)dh_gated; a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v;
+    a.f = (const float*)f; a.i = (const float*)i; a.o = (const float*)o;
+    a.dq = (float*)dq; a.dk = (float*)dk; a.dv = (float*)dv; a.df = (float*)df; a.di = (float*)di; a.d_o = (float*)d_o;
+    a.BH = B * NH; a.S = S; a.D = D;
+    return launch_scan_backward(a, (char*)sc.p, st, scan_mark);
 }
 
 }  // extern "C"

@@ -138,6 +138,13 @@ static int launch_df_t(const DfArgs& a, hipStream_t st) {
     return (int)hipGetLastError();
 }
 
+int launch_dfscan_plain(int gate_dtype, const void* F, const float* x, void* dF, int BH, int S, hipStream_t st) {
+    if (gate_dtype != MLSTM_F32) return MLSTM_ESHAPE;
+    hipLaunchKernelGGL(dfscan_kernel<float>, dim3(BH), dim3(1024), 0, st, reinterpret_cast<const float*>(F), x, reinterpret_cast<float*>(dF), S,
+                       1, 0, nullptr, 0);
+    return (int)hipGetLastError();
+}
+
 int launch_df(int gate_dtype, const DfArgs& a, hipStream_t st) {
     switch (gate_dtype) {
         case MLSTM_F32: return launch_df_t<float>(a, st);

@@ -161,9 +161,28 @@ struct ScanArgs {
     float* P;             // [BH, NC, 64, 64] in-chunk pair weights
     float* Nst;           // [BH, NC, D] vector state n~ at every chunk end
     int BH, S, D, NC;
+    // What the last kernel writes to h: 0 = silu(o) * numerator / n (the scan form's output), 1 = numerator / n (ungated),
+    // 2 = the numerator itself, sum_j exp(a_j - A_t) (q_t . k_j) / sqrt(D) v_j: the causal weighted sum the backward pass
+    // reuses with other operands in the places of q, k and v.  Bout (may be null): the normaliser sums b_t, modes 0 and 1.
+    int finish_mode;
+    float* Bout;
 };
 int scan_key_splits(int BH, int D);
 // mark(kernel id, stream, begin?) brackets groups of launches for the optional event timing
 int launch_scan(const ScanArgs& a, int KS, hipStream_t st, void (*mark)(int, hipStream_t, bool));
+// n~ at every chunk end from the chunks' own sums, in place (ScanArgs::Nst, beta2, G2, BH, NC, D are read)
+void launch_scan_ncarry(const ScanArgs& a, hipStream_t st);
+
+// Backward of the scan form (mlstm_scan_bwd.hip): every pointer fp32, [B,NH,S,D] or [B,NH,S]; ws holds
+// scan_backward_workspace_bytes(BH, S, D) bytes
+struct ScanBwdArgs {
+    const float* dhg; const float* q; const float* k; const float* v; const float* f; const float* i; const float* o;
+    float* dq; float* dk; float* dv; float* df; float* di; float* d_o;
+    int BH, S, D;
+};
+size_t scan_backward_workspace_bytes(int BH, int S, int D);
+int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*mark)(int, hipStream_t, bool));
+// dF_t = sigmoid(-f_t) * sum_{s<t} x_s over each head (x: [BH,S] fp32; dF_0 = 0): the scan of launch_df on its own
+int launch_dfscan_plain(int gate_dtype, const void* F, const float* x, void* dF, int BH, int S, hipStream_t st);
 
 }  // namespace mlstm

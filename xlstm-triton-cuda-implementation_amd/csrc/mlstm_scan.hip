@@ -357,16 +357,22 @@ __global__ __launch_bounds__(256) void scan_finish_kernel(ScanArgs a, int KS) {
         }
         const float prow = a.P[((size_t)bh * a.NC + c) * GRAN * GRAN + (size_t)(t - GRAN * c) * GRAN + lane];
         const float b = dot + wave_reduce<OpAdd>(prow);
-        const float inv = 1.0f / (fmaxf(fabsf(b), __expf(-a.M[row])) + 1e-6f);
+        const float inv = a.finish_mode == 2 ? 1.0f : 1.0f / (fmaxf(fabsf(b), __expf(-a.M[row])) + 1e-6f);
+        if (a.Bout && lane == 0) a.Bout[row] = b;
         for (int k = 4 * lane; k < D; k += 256) {
             f32x4 x = *reinterpret_cast<const f32x4*>(a.h + row * D + k);
             for (int p = 1; p < KS; p++) {
                 const f32x4 y = *reinterpret_cast<const f32x4*>(a.hpart + ((size_t)(p - 1) * rows + row) * D + k);
                 x += y;
             }
-            const f32x4 ov = *reinterpret_cast<const f32x4*>(a.o + row * D + k);
+            if (a.finish_mode == 0) {
+                const f32x4 ov = *reinterpret_cast<const f32x4*>(a.o + row * D + k);
 #pragma unroll
-            for (int e = 0; e < 4; e++) x[e] = x[e] * inv * (ov[e] / (1.0f + __expf(-ov[e])));
+                for (int e = 0; e < 4; e++) x[e] = x[e] * inv * (ov[e] / (1.0f + __expf(-ov[e])));
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) x[e] *= inv;
+            }
             *reinterpret_cast<f32x4*>(a.h + row * D + k) = x;
         }
     }
@@ -408,6 +414,10 @@ static int launch_scan_d(const ScanArgs& a, int KS, int NW, hipStream_t st, void
     hipLaunchKernelGGL(scan_finish_kernel, dim3(blocks), dim3(256), 0, st, a, KS);
     mark(MLSTM_K_SCAN_OUT, st, false);
     return (int)hipGetLastError();
+}
+
+void launch_scan_ncarry(const ScanArgs& a, hipStream_t st) {
+    hipLaunchKernelGGL(scan_ncarry_kernel, dim3((a.D + 255) / 256, a.BH), dim3(256), 0, st, a);
 }
 
 // Key ranges per value tile and waves per workgroup.
