@@ -226,20 +226,28 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
     return out, host
 
 
-def run_scan(ffi, steps, warmup):
-    """Scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape)."""
+def run_scan(ffi, steps, warmup, backward=False):
+    """Scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape); ``backward``: a step is the
+    forward followed by the backward (which recomputes the forward: five passes of the state kernel in all)."""
     L = ffi.lib()
     B, NH, S, D = 1, 4, 2048, 1024
     dev = torch.device("cuda:0")
     host = make_inputs(B, NH, S, D, torch.float32, 0.0, 0.0, 1.0, with_o=True)
-    q, k, v, f, i, _, o = (x.to(dev) for x in host)
+    q, k, v, f, i, dh, o = (x.to(dev) for x in host)
     h = torch.empty_like(q)
     ws, ws_n = ffi.workspace(ffi.OP_SCAN_FORWARD, B, NH, S, D, ffi.F32, dev)
     st, P = ffi.stream_ptr(), ffi.ptr
+    if backward:
+        dq, dk, dv, do = (torch.empty_like(q) for _ in range(4))
+        df, di = torch.empty_like(f), torch.empty_like(i)
+        wsb, wsb_n = ffi.workspace(ffi.OP_SCAN_BACKWARD, B, NH, S, D, ffi.F32, dev)
 
     def step():
         ffi.check_rc(L.mlstm_scan_forward_ex(P(q), P(k), P(v), P(f), P(i), P(o), P(h), B, NH, S, D, ffi.F32, P(ws), ws_n, st),
                      "mlstm_scan_forward_ex")
+        if backward:
+            ffi.check_rc(L.mlstm_scan_backward_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(o), P(dq), P(dk), P(dv), P(df), P(di), P(do),
+                                                  B, NH, S, D, ffi.F32, P(wsb), wsb_n, st), "mlstm_scan_backward_ex")
 
     for _ in range(warmup):
         step()
@@ -255,15 +263,18 @@ def run_scan(ffi, steps, warmup):
         step()
     torch.cuda.synchronize()
     ffi.timing_enable(False)
-    kern = {name: ffi.timing_read(name) for name in ("gates", "scan_carry", "scan_state", "scan_out")}
+    names = ("gates", "scan_carry", "scan_state", "scan_out") + (("scan_glue", "gate_bwd", "df") if backward else ())
+    kern = {name: ffi.timing_read(name) for name in names}
     ms_step = (t1 - t0) * 1e3 / steps
     BH = B * NH
-    bytes_compulsory = (5.0 * BH * S * D + 3.0 * BH * S) * 4          # q, k, v, o in, h out, f, i in (+ m)
+    # forward: q, k, v, o in, h out, f, i in (+ m); the backward adds dh in and six gradients out, and reads q, k, v, o, f, i again
+    bytes_compulsory = (5.0 * BH * S * D + 3.0 * BH * S) * 4 + (backward * (10.0 * BH * S * D + 4.0 * BH * S) * 4)
     flops = BH * (S / 64.0) * (2 * 64 * D * D * 2 + 2 * 2 * D * 64 * 65 / 2 * 2)  # state update + read-out, in-chunk pairs
-    st_ms = kern["scan_state"][0] / max(kern["scan_state"][1], 1)
+    st_ms = kern["scan_state"][0] / max(kern["scan_state"][1], 1)   # (average over the passes of a step)
     t_fl = flops / (st_ms * 1e-3) / 1e12 if st_ms else 0.0
+    flops *= 5 if backward else 1
     return {
-        "metric": "mLSTM scan-form forward, compulsory HBM GB/s, cfg3_B1_H4_S2048_D1024_f32",
+        "metric": "mLSTM scan-form %s, compulsory HBM GB/s, cfg3_B1_H4_S2048_D1024_f32" % ("forward+backward" if backward else "forward"),
         "value": bytes_compulsory / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
@@ -283,7 +294,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan"])
+    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan", "cfg3_scan_backward"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
@@ -306,8 +317,8 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if args.workload == "cfg3_scan":
-        print(json.dumps(run_scan(ffi, args.steps, args.warmup)))
+    if args.workload in ("cfg3_scan", "cfg3_scan_backward"):
+        print(json.dumps(run_scan(ffi, args.steps, args.warmup, backward=args.workload.endswith("backward"))))
         return
     out, host = run_matmul(ffi, args.workload, args.steps, args.warmup, precise=args.precise)
     headline = args.workload == "cfg4_B4_H8_S4096_D256_bf16" and not args.precise
@@ -315,7 +326,7 @@ def main():
         few = max(min(args.steps, 20), 5)
         out["secondary"] = [run_matmul(ffi, args.workload, few, 3, precise=True, host=host)[0],
                             run_matmul(ffi, "cfg5_B2_H32_S16384_D128_bf16", few, 3)[0],
-                            run_scan(ffi, max(args.steps, 20), 5)]
+                            run_scan(ffi, max(args.steps, 20), 5), run_scan(ffi, max(args.steps // 4, 10), 3, backward=True)]
     if not args.no_cpu_baseline:
         S, D = WORKLOADS[args.workload][2:4]
         out["cpu_baseline"] = cpu_baseline(host, S, D)
