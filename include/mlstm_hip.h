@@ -38,6 +38,30 @@ extern "C" {
  */
 #define MLSTM_PRECISE 0x100
 
+/*
+ * Layout of the caller's tensors, for the entry points that take one (names ending in _lx).  Element (b, h, s, d) of
+ * a [B,NH,S,D] tensor lies at  b * stride_b + h * stride_h + s * stride_s + d  elements from its base pointer: the
+ * head dimension is contiguous, everything else is free, so the [B,S,NH,D] activations of a projection (stride_b =
+ * S*NH*D, stride_h = D, stride_s = NH*D), or the q / k / v slices of one fused [B,S,3,NH,D] projection, are taken as
+ * they are, without the transposing copy the reference needs in front of its kernels (the step the reference's
+ * cutlass-src-hopper/mlstm_forward.cu:201 suggests fusing away).  One layout for q, k, v and their gradients, one for
+ * h and its gradient, one (without d) for the gates f, i and their gradients.  Rows must start on 16-byte boundaries:
+ * base pointers 16-byte aligned, qkv / out strides multiples of 8 elements (16-bit types) or 4 (fp32).
+ * gate_form says what `f` holds: the forget gate's pre-activation (the reference's input, mlstm_matmul.py:57), its
+ * log-sigmoid, or the cumulative sum of the log-sigmoid over the positions of each head (what mlstm_matmul.py:57-58
+ * compute first; fp32 gates only: the sum reaches 1e3..1e4 and 16-bit types cannot hold it).  The backward returns
+ * in `df` the gradient of whatever `f` held.  m and b (statistics) are always dense [B,NH,S] fp32.
+ */
+#define MLSTM_GATE_RAW 0
+#define MLSTM_GATE_LOGSIGMOID 1
+#define MLSTM_GATE_CUMSUM 2
+typedef struct mlstm_layout {
+    long long qkv_stride_b, qkv_stride_h, qkv_stride_s;
+    long long out_stride_b, out_stride_h, out_stride_s;
+    long long gate_stride_b, gate_stride_h, gate_stride_s;
+    int gate_form;
+} mlstm_layout;
+
 /* argument errors */
 #define MLSTM_EINVAL (-1)      /* null pointer, non-positive size, unknown dtype */
 #define MLSTM_ESHAPE (-2)      /* head dimension / sequence length not supported by this build */
@@ -124,6 +148,30 @@ int mlstm_backward_saved_ex(const void* dh, const void* q, const void* k, const 
                             const void* h, const float* m, const float* b, const void* saved, size_t saved_bytes,
                             void* dq, void* dk, void* dv, void* df, void* di, int B, int NH, int S, int D, int dtype,
                             int gate_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * The four entry points above for tensors in a layout of the caller's (see mlstm_layout; null = dense, which makes
+ * each identical to its _ex namesake): the activations of a [B,S,NH,D] projection, or the slices of a fused q/k/v
+ * projection, go in without a transposing copy, the forget gate may come as its log-sigmoid or as the cumulative sum
+ * of that, and h, dq, dk, dv, df, di are written in the same layouts.  The kernels address rows through the layout's
+ * strides; nothing else changes, and results are bit-identical to a run on dense copies.  No counterpart in the
+ * reference, whose kernels take contiguous [B,NH,S,D] only (mlstm_matmul.py:121-129, :368-405); the hint to take the
+ * step before the kernel into it is at cutlass-src-hopper/mlstm_forward.cu:201.
+ */
+int mlstm_forward_lx(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
+                     int B, int NH, int S, int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace,
+                     size_t workspace_bytes, void* stream);
+int mlstm_backward_lx(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
+                      const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, int B, int NH, int S,
+                      int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace, size_t workspace_bytes,
+                      void* stream);
+int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
+                          void* saved, size_t saved_bytes, int B, int NH, int S, int D, int dtype, int gate_dtype,
+                          const mlstm_layout* layout, void* workspace, size_t workspace_bytes, void* stream);
+int mlstm_backward_saved_lx(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
+                            const float* m, const float* b, const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv,
+                            void* df, void* di, int B, int NH, int S, int D, int dtype, int gate_dtype, const mlstm_layout* layout,
+                            void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Matmul form with the output gate of the scan form, h_gated = silu(o) * h (mlstm_scan.py:277): the item the

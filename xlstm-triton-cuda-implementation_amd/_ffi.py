@@ -17,6 +17,15 @@ _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dty
            -3: "workspace (or saved buffer) too small or of the wrong size",
            -4: "a kernel's bounded wait expired"}
 
+GATE_FORMS = {"raw": 0, "logsigmoid": 1, "cumsum": 2}   # MLSTM_GATE_RAW / _LOGSIGMOID / _CUMSUM
+
+
+class Layout(ctypes.Structure):
+    """struct mlstm_layout: element strides (batch, head, position) of q/k/v, of h/dh and of the gates; what f holds."""
+    _fields_ = [(n, ctypes.c_longlong) for n in ("qkv_b", "qkv_h", "qkv_s", "out_b", "out_h", "out_s", "gate_b", "gate_h", "gate_s")] + \
+               [("gate_form", ctypes.c_int)]
+
+
 _lib = None
 
 
@@ -53,6 +62,15 @@ def lib():
         L.mlstm_forward_gated_ex.argtypes = [vp] * 10 + [ci] * 6 + [vp, sz, vp]
         L.mlstm_backward_gated_ex.restype = ci
         L.mlstm_backward_gated_ex.argtypes = [vp] * 16 + [ci] * 6 + [vp, sz, vp]
+        lp = ctypes.POINTER(Layout)
+        L.mlstm_forward_lx.restype = ci
+        L.mlstm_forward_lx.argtypes = [vp] * 8 + [ci] * 6 + [lp, vp, sz, vp]
+        L.mlstm_backward_lx.restype = ci
+        L.mlstm_backward_lx.argtypes = [vp] * 14 + [ci] * 6 + [lp, vp, sz, vp]
+        L.mlstm_forward_save_lx.restype = ci
+        L.mlstm_forward_save_lx.argtypes = [vp] * 9 + [sz] + [ci] * 6 + [lp, vp, sz, vp]
+        L.mlstm_backward_saved_lx.restype = ci
+        L.mlstm_backward_saved_lx.argtypes = [vp] * 10 + [sz] + [vp] * 5 + [ci] * 6 + [lp, vp, sz, vp]
         L.mlstm_scan_forward_ex.restype = ci
         L.mlstm_scan_forward_ex.argtypes = [vp] * 7 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_scan_backward_ex.restype = ci
@@ -79,7 +97,7 @@ def lib():
 
 def exported_symbols():
     return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
-            "mlstm_scan_backward_ex",
+            "mlstm_scan_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
@@ -139,6 +157,49 @@ def require(t, name, shape=None):
         raise ValueError(f"{name} must be contiguous")
     if shape is not None and tuple(t.shape) != tuple(shape):
         raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def require_rows(t, name, shape=None, like=None):
+    """A GPU tensor whose last dimension is contiguous (any strides elsewhere: the kernels address rows through them)."""
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got device {t.device})")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    if t.dim() == 4 and t.stride(-1) != 1 and t.shape[-1] > 1:
+        raise ValueError(f"{name}: the head dimension must be contiguous (strides {t.stride()})")
+    if like is not None and tuple(t.stride()) != tuple(like.stride()):
+        raise ValueError(f"{name} must have the layout of its companion (strides {t.stride()} against {like.stride()})")
+
+
+def dense_in_order_of(t):
+    """A new tensor of t's shape, contiguous in the order of t's dimensions in memory (for a [B,NH,S,D] view of
+    [B,S,NH,D] activations that is again such a view)."""
+    order = sorted(range(t.dim()), key=lambda d: (t.stride(d), -d if t.shape[d] == 1 else 0), reverse=True)
+    if t.dim() == 4:
+        order = [d for d in order if d != 3] + [3]
+    buf = torch.empty([t.shape[d] for d in order], dtype=t.dtype, device=t.device)
+    inverse = [order.index(d) for d in range(t.dim())]
+    return buf.permute(inverse)
+
+
+def span(t):
+    return 1 + sum((n - 1) * s for n, s in zip(t.shape, t.stride())) if t.numel() else 0
+
+
+def strided_like(t, count=1):
+    """`count` new tensors with exactly t's shape and strides."""
+    if t.is_contiguous() or torch._prims_common.is_non_overlapping_and_dense(t):
+        return [torch.empty_strided(t.shape, t.stride(), dtype=t.dtype, device=t.device) for _ in range(count)]
+    n = span(t)
+    return [torch.empty(n, dtype=t.dtype, device=t.device).as_strided(t.shape, t.stride()) for _ in range(count)]
+
+
+def layout(q, h, f, gate_form="raw"):
+    """struct mlstm_layout for q (and k, v, dq, dk, dv), h (and dh) and f (and i, df, di), all [B,NH,S(,D)] views."""
+    if gate_form not in GATE_FORMS:
+        raise ValueError(f"gate_form must be one of {sorted(GATE_FORMS)}, got {gate_form!r}")
+    return Layout(q.stride(0), q.stride(1), q.stride(2), h.stride(0), h.stride(1), h.stride(2),
+                  f.stride(0), f.stride(1), f.stride(2), GATE_FORMS[gate_form])
 
 
 def ptr(t):

@@ -72,6 +72,10 @@ struct Sizes {
         return up256(BH * n * D * D * 4) + up256(BH * n * D * D * el) + up256(BH * n * D * 4);
     }
     int dtype_code = MLSTM_F32;
+    // layouts of the caller's tensors (dense unless an _lx entry point says otherwise): q, k, v and their gradients;
+    // h and dh; the gates and their gradients; and what f holds
+    Lay la{}, lb{}, lg{};
+    int gate_form = MLSTM_GATE_RAW;
     bool precise = false;   // split mode (MLSTM_PRECISE): no chunks, and the low-order part of h travels to the backward
     int chunk_len() const { return chunk_len_for(dtype_code, (int)D, S, precise); }
     size_t states_t() const { return up256(BH * n_states(chunk_len()) * D * D * el); }   // value-major copy for the dQ pass
@@ -115,9 +119,32 @@ Sizes sizes_of(int B, int NH, int S, int D, int dtype_arg) {
     const int dt = dtype_arg & ~MLSTM_PRECISE;
     Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, dtype_size(dt), dt};
     z.precise = precise_of(dtype_arg);
+    z.la = z.lb = dense_layout(NH, S, D);
+    z.lg = dense_layout(NH, S, 1);
     return z;
 }
 bool good_shape(int D, int dtype) { return D == 64 || D == 128 || (D == 256 && dtype != MLSTM_F32); }
+
+// The caller's layout into z (null: everything dense).  Rows of q, k, v, h must start on 16-byte boundaries, and the
+// tile copies address a tile's 64 rows with 32-bit byte offsets.
+int apply_layout(Sizes& z, const mlstm_layout* L, int NH, int gate_dtype, std::initializer_list<const void*> row_tensors) {
+    if (!L) return 0;
+    const long long el = (long long)z.el;
+    auto good = [&](long long b, long long h, long long s) {
+        return b >= 0 && h >= 0 && s >= (long long)z.D && (b * el) % 16 == 0 && (h * el) % 16 == 0 && (s * el) % 16 == 0 && s * el <= (1ll << 24);
+    };
+    if (!good(L->qkv_stride_b, L->qkv_stride_h, L->qkv_stride_s) || !good(L->out_stride_b, L->out_stride_h, L->out_stride_s)) return MLSTM_EINVAL;
+    if (L->gate_stride_b < 0 || L->gate_stride_h < 0 || L->gate_stride_s < 1) return MLSTM_EINVAL;
+    if (L->gate_form != MLSTM_GATE_RAW && L->gate_form != MLSTM_GATE_LOGSIGMOID && L->gate_form != MLSTM_GATE_CUMSUM) return MLSTM_EINVAL;
+    if (L->gate_form == MLSTM_GATE_CUMSUM && gate_dtype != MLSTM_F32) return MLSTM_EINVAL;
+    for (const void* p : row_tensors)
+        if (p && (reinterpret_cast<size_t>(p) & 15)) return MLSTM_EINVAL;
+    z.la = Lay{L->qkv_stride_b, L->qkv_stride_h, L->qkv_stride_s, NH};
+    z.lb = Lay{L->out_stride_b, L->out_stride_h, L->out_stride_s, NH};
+    z.lg = Lay{L->gate_stride_b, L->gate_stride_h, L->gate_stride_s, NH};
+    z.gate_form = L->gate_form;
+    return 0;
+}
 
 // RAII for a stream-ordered scratch allocation when the caller brings no workspace
 struct Scratch {
@@ -209,6 +236,7 @@ int chunk_states_impl(const void* k, const void* v, const FwdWs& w, bool key_maj
                       hipStream_t st) {
     ChunkArgs ca{k, v, w.alpha2, w.beta2, w.G2, w.dC, Nst, key_major ? w.Cst : nullptr, CstT, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs,
                  0, nullptr, nullptr};
+    ca.lk = ca.lv = z.la;
     Timed t(MLSTM_K_CHUNK_STATES, st);
     return launch_chunk_states(dtype, D, ca, st);
 }
@@ -226,10 +254,11 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
     if (!b) b = w.bw;
     {
         Timed t(MLSTM_K_GATES, st);
-        hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st);
+        hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st, z.lg, z.gate_form);
         if (e != hipSuccess) return (int)e;
     }
     RowArgs a{};
+    a.la = z.la; a.lb = z.lb; a.lh = z.lb;
     a.X = q; a.Y1 = k; a.Y2 = v; a.out = h; a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.Bsum = b;
     a.ek2 = ek2; a.amax2 = amax2; a.O = o; a.out_gated = h_gated;
     a.BH = (int)z.BH; a.S = (int)z.S; a.NG = (int)z.NG;
@@ -346,13 +375,20 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype) {
 int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                      int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes,
                      void* stream) {
+    return mlstm_forward_lx(q, k, v, f, i, h, m, b, B, NH, S, D, dtype, gate_dtype, nullptr, workspace, workspace_bytes, stream);
+}
+
+int mlstm_forward_lx(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
+                     int B, int NH, int S, int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace,
+                     size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
     const int dtype_arg = dtype;
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h})) return rc;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -384,13 +420,21 @@ size_t mlstm_saved_state_bytes(int B, int NH, int S, int D, int dtype) {
 int mlstm_forward_save_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                           void* saved, size_t saved_bytes, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace,
                           size_t workspace_bytes, void* stream) {
+    return mlstm_forward_save_lx(q, k, v, f, i, h, m, b, saved, saved_bytes, B, NH, S, D, dtype, gate_dtype, nullptr, workspace,
+                                 workspace_bytes, stream);
+}
+
+int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
+                          void* saved, size_t saved_bytes, int B, int NH, int S, int D, int dtype, int gate_dtype,
+                          const mlstm_layout* layout, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !f || !i || !h || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
     const int dtype_arg = dtype;
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h})) return rc;
     if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
@@ -454,6 +498,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     // (saved), or the forward is run again here
     const void* h_lo = z.precise ? saved : nullptr;
     const bool have_fwd = h && m && b && (!z.precise || h_lo);
+    Lay lh = z.lb;   // layout of the forward output the dQ pass reads
     if (have_fwd) {
         // gates only: alpha, beta, G (and m again, into the workspace) are cheap to rebuild; so are the chunk states
         G2 = w.G2; alpha2 = w.alpha2; beta2 = w.beta2; ek2 = w.ek2; amax2 = w.amax2; mm = w.mw;
@@ -461,14 +506,16 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
             mm = const_cast<float*>(m);
         } else {
             Timed t(MLSTM_K_GATES, st);
-            hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, mm, ek2, amax2, (int)z.BH, (int)z.S, st);
+            hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, mm, ek2, amax2, (int)z.BH, (int)z.S, st, z.lg, z.gate_form);
             if (e != hipSuccess) return (int)e;
         }
         bb = const_cast<float*>(b);
         if (w.ncs > 0 && !saved)
             if (int e = chunk_states_impl(k, v, w, false, CstT, w.Nst, z, D, dtype, st)) return e;   // (the dQ pass wants them value-major only)
     } else {
-        int rc = forward_impl(q, k, v, f, i, hbuf, nullptr, nullptr, z, D, dtype, gate_dtype, ws, st, &alpha2, &beta2, &G2, &mm, &bb, &ek2, &amax2,
+        Sizes zf = z;            // (the recomputed h is the library's own, dense)
+        zf.lb = lh = dense_layout(z.la.NH, (long long)z.S, (long long)z.D);
+        int rc = forward_impl(q, k, v, f, i, hbuf, nullptr, nullptr, zf, D, dtype, gate_dtype, ws, st, &alpha2, &beta2, &G2, &mm, &bb, &ek2, &amax2,
                               nullptr, nullptr, CstT, nullptr, nullptr, z.precise ? hlo_buf : nullptr);
         Nst = w.Nst;
         if (rc) return rc;
@@ -477,6 +524,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     }
     // dQ first: it derives 1/n and db per row from (dh, h, m, b) and leaves them for the column kernel
     RowArgs ra{};
+    ra.la = z.la; ra.lb = z.lb; ra.lh = lh;
     ra.X = dh; ra.Y1 = v; ra.Y2 = k; ra.out = dq; ra.alpha2 = alpha2; ra.beta2 = beta2; ra.G2 = G2; ra.inv_n = inv_n; ra.db = dbuf;
     ra.ek2 = ek2; ra.amax2 = amax2; ra.Hin = h; ra.Bin = bb; ra.M = mm;
     ra.BH = (int)z.BH; ra.S = (int)z.S; ra.NG = (int)z.NG;
@@ -493,10 +541,12 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         // itself), and the dF anchors at the chunk boundaries
         Timed t(MLSTM_K_CHUNK_STATES, st);
         ChunkArgs ra2{q, dh, alpha2, beta2, G2, w.dC, gvec, nullptr, Ev, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs, 1, inv_n, dbuf};
+        ra2.lk = z.la; ra2.lv = z.lb;
         if (int e = launch_chunk_states(dtype, D, ra2, st)) return e;
         if (int e = launch_anchor(dtype, D, CstT, Ev, Nst, gvec, anchor, (int)z.BH, (int)w.ncs, st)) return e;   // (both value-major)
     }
     ColArgs ca{};
+    ca.la = z.la; ca.lb = z.lb;
     ca.Q = q; ca.K = k; ca.V = v; ca.dH = dh; ca.dK = dk; ca.dV = dv; ca.colsum = colsum; ca.rowpart = rowpart;
     ca.alpha2 = alpha2; ca.beta2 = beta2; ca.G2 = G2; ca.inv_n = inv_n; ca.db = dbuf;
     ca.BH = (int)z.BH; ca.S = (int)z.S; ca.NG = (int)z.NG;
@@ -508,6 +558,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     }
 
     DfArgs da{f, colsum, rowpart, df, di, (int)z.BH, (int)z.S, (int)z.NG, (int)z.row_slices(), col_chunks ? w.L : 0, rowinter, anchor, (int)w.ncs};
+    da.lg = z.lg; da.gate_form = z.gate_form;
     Timed t(MLSTM_K_DF, st);
     return launch_df(gate_dtype, da, st);
 }
@@ -519,6 +570,13 @@ extern "C" {
 int mlstm_backward_ex(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
                       const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, int B, int NH, int S,
                       int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return mlstm_backward_lx(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, B, NH, S, D, dtype, gate_dtype, nullptr, workspace, workspace_bytes,
+                             stream);
+}
+
+int mlstm_backward_lx(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
+                      const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, int B, int NH, int S,
+                      int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace, size_t workspace_bytes, void* stream) {
     if (!dh || !q || !k || !v || !f || !i || !dq || !dk || !dv || !df || !di || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) ||
         !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
@@ -526,7 +584,8 @@ int mlstm_backward_ex(const void* dh, const void* q, const void* k, const void* 
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv})) return rc;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;
     return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -536,6 +595,14 @@ int mlstm_backward_saved_ex(const void* dh, const void* q, const void* k, const 
                             const float* m, const float* b, const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv, void* df,
                             void* di, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes,
                             void* stream) {
+    return mlstm_backward_saved_lx(dh, q, k, v, f, i, h, m, b, saved, saved_bytes, dq, dk, dv, df, di, B, NH, S, D, dtype, gate_dtype, nullptr,
+                                   workspace, workspace_bytes, stream);
+}
+
+int mlstm_backward_saved_lx(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h,
+                            const float* m, const float* b, const void* saved, size_t saved_bytes, void* dq, void* dk, void* dv, void* df,
+                            void* di, int B, int NH, int S, int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace,
+                            size_t workspace_bytes, void* stream) {
     if (!dh || !q || !k || !v || !f || !i || !h || !m || !b || !dq || !dk || !dv || !df || !di || B <= 0 || NH <= 0 || S <= 0 ||
         !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
@@ -543,7 +610,8 @@ int mlstm_backward_saved_ex(const void* dh, const void* q, const void* k, const 
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv})) return rc;
     if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;

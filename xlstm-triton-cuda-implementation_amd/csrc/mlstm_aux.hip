@@ -12,7 +12,7 @@ namespace mlstm {
 // slices at or below the position's own tile), the four partial sums meet in LDS.
 template <typename TG>
 __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict__ colsum, float* rowpart, TG* __restrict__ dI,
-                                                        int S, int NG, int RS, int chunk_tiles, const float* __restrict__ rowinter) {
+                                                        int S, int NG, int RS, int chunk_tiles, const float* __restrict__ rowinter, Lay lg) {
     __shared__ float part[4][GRAN];
     const int bh = blockIdx.y, g = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = GRAN * g + lane, tc = t < S ? t : S - 1;
@@ -35,8 +35,17 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict_
         const float col = colsum[(size_t)bh * S + t];
         const float row = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]) + (rowinter ? rowinter[(size_t)bh * S + t] : 0.f);
         rowpart[(size_t)bh * RS * S + t] = col - row;
-        dI[(size_t)bh * S + t] = (TG)col;
+        dI[lg.head(bh) + (size_t)t * lg.ss] = (TG)col;
     }
+}
+
+// The gradient of what the caller's F holds (DfArgs::gate_form) from the running sum excl_t = sum_{s<t} x_s and x_t itself:
+// the pre-activation sees it through the log-sigmoid's derivative sigmoid(-f); the log-sigmoid lf_t takes it as it is;
+// the cumulative sum Fc (lf_t = Fc_t - Fc_{t-1}) gets excl_t - excl_{t+1} = -x_t, at every position.
+__device__ __forceinline__ float forget_grad(int form, float f, float excl, float x, int t) {
+    if (form == MLSTM_GATE_CUMSUM) return -x;
+    if (t == 0) return 0.f;
+    return form == MLSTM_GATE_RAW ? excl / (1.0f + __expf(f)) : excl;
 }
 
 // In chunks the running sum is re-anchored at every chunk start: sum_{s<t} (col_s - row_s) is the sum of dD over the pairs
@@ -45,7 +54,8 @@ __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict_
 // position's sum is off by some 2^-9 of its size, independently, and a plain running sum would add those up).
 template <typename TG>
 __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, const float* __restrict__ rowpart, TG* __restrict__ dF,
-                                                      int S, int RS, int chunk_len, const float* __restrict__ anchor, int n_states) {
+                                                      int S, int RS, int chunk_len, const float* __restrict__ anchor, int n_states, Lay lg,
+                                                      int form) {
     __shared__ float wt[2][16];
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const float* x = rowpart + (size_t)bh * RS * S;
@@ -56,7 +66,7 @@ __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, 
         if (chunk_len > 0 && base > 0 && base % chunk_len == 0) carry = (double)anchor[(size_t)bh * n_states + base / chunk_len - 1];
         const int t = base + tid;
         const float v = t < S && tid < step ? x[t] : 0.f;
-        const float f = t < S ? (float)F[(size_t)bh * S + t] : 0.f;
+        const float f = t < S ? (float)F[lg.head(bh) + (size_t)t * lg.ss] : 0.f;
         const float incl = wave_scan_inclusive<OpAdd>(v);
         if (lane == 63) wt[par][wave] = incl;
         __syncthreads();  // (the totals alternate between two buffers: one barrier per block of 1024 positions)
@@ -73,9 +83,8 @@ __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, 
         if (chunk_len > 0 && step == chunk_len && base / chunk_len < n_states)
             bridge = (float)((double)anchor[(size_t)bh * n_states + base / chunk_len] - (carry + (double)tot)) / (float)step;
         if (t < S && tid < step) {
-            const float sg = 1.0f / (1.0f + __expf(f));  // sigmoid(-f)
             const float excl = (float)(carry + (double)(pre + (incl - v))) + bridge * (float)tid;
-            dF[(size_t)bh * S + t] = (TG)(t == 0 ? 0.f : sg * excl);
+            dF[lg.head(bh) + (size_t)t * lg.ss] = (TG)forget_grad(form, f, excl, v, t);
         }
         carry += (double)tot;
     }
@@ -87,7 +96,8 @@ __global__ __launch_bounds__(1024) void dfscan_kernel(const TG* __restrict__ F, 
 template <typename TG>
 __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F, const float* __restrict__ colsum, const float* __restrict__ rowpart,
                                                        const float* __restrict__ rowinter, const float* __restrict__ anchor,
-                                                       TG* __restrict__ dF, TG* __restrict__ dI, int S, int RS, int chunk_len, int n_states) {
+                                                       TG* __restrict__ dF, TG* __restrict__ dI, int S, int RS, int chunk_len, int n_states,
+                                                       Lay lg, int form) {
     __shared__ float wt[16];
     const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int t = c * chunk_len + tid;
@@ -99,7 +109,7 @@ __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F,
         float row = rowinter[(size_t)bh * S + t];
         for (int j = g0; j <= g; j++) row += rp[(size_t)(j - g0) * S];
         col = colsum[(size_t)bh * S + t];
-        f = (float)F[(size_t)bh * S + t];
+        f = (float)F[lg.head(bh) + (size_t)t * lg.ss];
         v = col - row;
     }
     const float incl = wave_scan_inclusive<OpAdd>(v);
@@ -116,10 +126,9 @@ __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F,
     // what the chunk's own (rounded) sums miss of the next anchor is spread evenly over its positions
     const float bridge = c < n_states ? (anchor[(size_t)bh * n_states + c] - (start + tot)) / (float)chunk_len : 0.f;
     if (live) {
-        const float sg = 1.0f / (1.0f + __expf(f));  // sigmoid(-f)
         const float excl = start + (pre + (incl - v)) + bridge * (float)tid;
-        dF[(size_t)bh * S + t] = (TG)(t == 0 ? 0.f : sg * excl);
-        dI[(size_t)bh * S + t] = (TG)col;
+        dF[lg.head(bh) + (size_t)t * lg.ss] = (TG)forget_grad(form, f, excl, v, t);
+        dI[lg.head(bh) + (size_t)t * lg.ss] = (TG)col;
     }
 }
 
@@ -128,20 +137,20 @@ static int launch_df_t(const DfArgs& a, hipStream_t st) {
     if (a.chunk_len > 0 && a.chunk_len <= 1024) {
         hipLaunchKernelGGL(dfchunk_kernel<TG>, dim3((a.S + a.chunk_len - 1) / a.chunk_len, a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F),
                            a.colsum, a.rowpart, a.rowinter, a.anchor, reinterpret_cast<TG*>(a.dF), reinterpret_cast<TG*>(a.dI), a.S, a.RS,
-                           a.chunk_len, a.n_states);
+                           a.chunk_len, a.n_states, a.lg, a.gate_form);
         return (int)hipGetLastError();
     }
     hipLaunchKernelGGL(rowreduce_kernel<TG>, dim3((a.S + GRAN - 1) / GRAN, a.BH), dim3(256), 0, st, a.colsum, const_cast<float*>(a.rowpart),
-                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.RS, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr);
+                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.RS, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr, a.lg);
     hipLaunchKernelGGL(dfscan_kernel<TG>, dim3(a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F), a.rowpart,
-                       reinterpret_cast<TG*>(a.dF), a.S, a.RS, a.chunk_len, a.anchor, a.n_states);
+                       reinterpret_cast<TG*>(a.dF), a.S, a.RS, a.chunk_len, a.anchor, a.n_states, a.lg, a.gate_form);
     return (int)hipGetLastError();
 }
 
 int launch_dfscan_plain(int gate_dtype, const void* F, const float* x, void* dF, int BH, int S, hipStream_t st) {
     if (gate_dtype != MLSTM_F32) return MLSTM_ESHAPE;
     hipLaunchKernelGGL(dfscan_kernel<float>, dim3(BH), dim3(1024), 0, st, reinterpret_cast<const float*>(F), x, reinterpret_cast<float*>(dF), S,
-                       1, 0, nullptr, 0);
+                       1, 0, nullptr, 0, dense_layout(BH, S, 1), MLSTM_GATE_RAW);
     return (int)hipGetLastError();
 }
 

@@ -74,11 +74,14 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     // forward states: sum cc is over chunk cc, relative to its own last position; reverse states (K = Q, V = dH): sum cc
     // is over chunk cc + 1 (the last chunk may be short), relative to the last position of chunk cc
     const int p0 = (a.reverse ? cc + 1 : cc) * L, pe = a.reverse ? p0 - 1 : p0 + L - 1;
-    const T* Kh = reinterpret_cast<const T*>(a.K) + (hoff + p0) * D;
-    const T* Vh = reinterpret_cast<const T*>(a.V) + (hoff + p0) * D + VW * vh;
+    // K and V are the caller's tensors, each in its layout (elements per position rsK / rsV)
+    const size_t rsK = (size_t)a.lk.ss, rsV = (size_t)a.lv.ss;
+    const T* Kh = reinterpret_cast<const T*>(a.K) + a.lk.head(bh) + (size_t)p0 * rsK;
+    const T* Vh = reinterpret_cast<const T*>(a.V) + a.lv.head(bh) + (size_t)p0 * rsV + VW * vh;
 
     TileDma<T, D, GRAN, 256> kdma;   // K tiles by direct loads; every position of a complete chunk exists
     kdma.init(tid);
+    const auto rk = kdma.rows(tid, (unsigned)(rsK * sizeof(T)));
     SwzTransReader<T, D> krd;        // per-lane offsets of the transposing reads, computed once
     krd.init(lane, (D / 128) * wave);
     SwzTransReader<T, VW> vrd;
@@ -101,13 +104,13 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     auto issue = [&](auto par_tag, int j) {   // loads of tile j: K into stage j % 3, V into the registers
         constexpr int P = decltype(par_tag)::value;
         T* kst = reinterpret_cast<T*>(ks + (j % ST) * Cfg::K_BYTES);
-        if (p0 + GRAN * (j + 1) <= S) kdma.issue(kst, Kh + (size_t)GRAN * j * D);
-        else tile_dma<T, D, GRAN, 256>(kst, Kh - (size_t)p0 * D, p0 + GRAN * j, S, tid);   // rows past the end are clamped (their weights are 0)
+        if (p0 + GRAN * (j + 1) <= S) kdma.issue(kst, Kh + (size_t)GRAN * j * rsK, rk);
+        else tile_dma<T, D, GRAN, 256>(kst, Kh - (size_t)p0 * rsK, p0 + GRAN * j, S, tid, rsK);   // rows past the end are clamped (their weights are 0)
 #pragma unroll
         for (int it = 0; it < 4; it++) {
             int pos = GRAN * j + vrow + 16 * it;
             pos = p0 + pos < S ? pos : S - 1 - p0;
-            gload16(vset[P][it], Vh + (size_t)pos * D + 8 * vch);
+            gload16(vset[P][it], Vh + (size_t)pos * rsV + 8 * vch);
         }
     };
     auto commit = [&](auto par_tag, int j) {  // V of tile j, times the positions' weights, into stage j % 3

@@ -83,27 +83,30 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
     const int kbA = wave >> 1, qbA = wave & 1;   // phase A block
     const int kbB = wave & 1, dsel = wave >> 1;  // phase B: keys 32*kbB.., column blocks dsel, dsel+2, ...
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN;
-    const T* Q = reinterpret_cast<const T*>(a.Q) + hoff * D;
-    const T* dH = reinterpret_cast<const T*>(a.dH) + hoff * D;
-    const T* K = reinterpret_cast<const T*>(a.K) + hoff * D;
-    const T* V = reinterpret_cast<const T*>(a.V) + hoff * D;
+    // the caller's tensors: q, k, v, dk, dv in layout la, dh in lb (element offset of the head, elements per position)
+    const size_t rsA = (size_t)a.la.ss, rsB = (size_t)a.lb.ss, offA = a.la.head(bh), offB = a.lb.head(bh);
+    const T* Q = reinterpret_cast<const T*>(a.Q) + offA;
+    const T* dH = reinterpret_cast<const T*>(a.dH) + offB;
+    const T* K = reinterpret_cast<const T*>(a.K) + offA;
+    const T* V = reinterpret_cast<const T*>(a.V) + offA;
     const float* const beta_head = a.beta2 + poff;
     const float* const inv_head = a.inv_n + poff;
     const float* const db_head = a.db + poff;
 
     TileDma<T, D, GRAN, 256> tdma;
     tdma.init(tid);
+    const auto ra = tdma.rows(tid, (unsigned)(rsA * sizeof(T))), rb = tdma.rows(tid, (unsigned)(rsB * sizeof(T)));
     RowVec3Dma rvdma;   // beta, 1/n, db of a query tile (padded arrays: always readable)
     rvdma.init(tid, beta_head, inv_head, db_head);
     const int full_tiles = S / GRAN;  // query tiles whose 64 rows all exist
 #define COL_DMA(it, st)                                                          \
     do {                                                                         \
         if ((it) < full_tiles) {                                                 \
-            tdma.issue(ST_Q(st), Q + (size_t)GRAN * (it) * D);                    \
-            tdma.issue(ST_DH(st), dH + (size_t)GRAN * (it) * D);                  \
+            tdma.issue(ST_Q(st), Q + (size_t)GRAN * (it) * rsA, ra);              \
+            tdma.issue(ST_DH(st), dH + (size_t)GRAN * (it) * rsB, rb);            \
         } else {                                                                 \
-            tile_dma<T, D, GRAN, 256>(ST_Q(st), Q, GRAN * (it), S, tid);          \
-            tile_dma<T, D, GRAN, 256>(ST_DH(st), dH, GRAN * (it), S, tid);        \
+            tile_dma<T, D, GRAN, 256>(ST_Q(st), Q, GRAN * (it), S, tid, rsA);     \
+            tile_dma<T, D, GRAN, 256>(ST_DH(st), dH, GRAN * (it), S, tid, rsB);   \
         }                                                                        \
         rvdma.issue(ST_ROW(st), (it));                                            \
     } while (0)
@@ -118,8 +121,8 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
     frag kf[NS], vf[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
-        kf[s] = frag_rowmajor<T>(K + (size_t)keyAc * D, s, h);
-        vf[s] = frag_rowmajor<T>(V + (size_t)keyAc * D, s, h);
+        kf[s] = frag_rowmajor<T>(K + (size_t)keyAc * rsA, s, h);
+        vf[s] = frag_rowmajor<T>(V + (size_t)keyAc * rsA, s, h);
     }
     float al[16];
 #pragma unroll
@@ -200,8 +203,8 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                 if (it + 1 < NG) { if (stage) COL_DMA(it + 1, 0); else COL_DMA(it + 1, 1); }
             }
         }
-        const T* gq = Q + (size_t)GRAN * (it + 1) * D;
-        const T* gdh = dH + (size_t)GRAN * (it + 1) * D;
+        const T* gq = Q + (size_t)GRAN * (it + 1) * rsA;
+        const T* gdh = dH + (size_t)GRAN * (it + 1) * rsB;
         T* const lq = ST_Q(stn);
         T* const ldh = ST_DH(stn);
         const T* Qs = ST_Q(stage);
@@ -225,7 +228,7 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
 #pragma unroll
             for (int s = 0; s < NS; s++) {
                 if constexpr (SPREAD && STAGES == 2) {
-                    if (s % AHEAD == 0) tdma.issue_range(lq, gq, (s / AHEAD) * PW / (NS / AHEAD), (s / AHEAD + 1) * PW / (NS / AHEAD));
+                    if (s % AHEAD == 0) tdma.issue_range(lq, gq, (s / AHEAD) * PW / (NS / AHEAD), (s / AHEAD + 1) * PW / (NS / AHEAD), ra);
                 }
                 if (s + AHEAD < NS) { qf[s + AHEAD] = qrd.read(Qs, qbA, s + AHEAD); hf[s + AHEAD] = qrd.read(dHs, qbA, s + AHEAD); }
                 if (s == 0) {
@@ -330,7 +333,7 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
         for (int x = 0; x < NXW; x++) read_qh(0, x);
 #pragma unroll
         for (int t = 0; t < NQS; t++) {
-            if constexpr (SPREAD && STAGES == 2) tdma.issue_range(ldh, gdh, t * PW / NQS, (t + 1) * PW / NQS);
+            if constexpr (SPREAD && STAGES == 2) tdma.issue_range(ldh, gdh, t * PW / NQS, (t + 1) * PW / NQS, rb);
 #pragma unroll
             for (int x = 0; x < NXW; x++) {
 #pragma unroll
@@ -391,12 +394,12 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                         *reinterpret_cast<typename R::vec4*>(stage + (32 * (BOTH_KB ? kb : kbB) + c32) * RB + d * (int)sizeof(T)) = R::cvt4(v);
                     }
             __syncthreads();
-            char* const gout = reinterpret_cast<char*>(which ? a.dV : a.dK) + (hoff + (size_t)GRAN * jt) * D * sizeof(T);
+            char* const gout = reinterpret_cast<char*>(which ? a.dV : a.dK) + (offA + (size_t)GRAN * jt * rsA) * sizeof(T);
 #pragma unroll
             for (int i = 0; i < GRAN * CPR / 256; i++) {
                 const int c = tid + 256 * i, row = c / CPR, cc = c % CPR;
                 if (GRAN * jt + row < S)
-                    *reinterpret_cast<uint4*>(gout + (size_t)row * D * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + row * RB + 16 * cc);
+                    *reinterpret_cast<uint4*>(gout + (size_t)row * rsA * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + row * RB + 16 * cc);
             }
         }
     }

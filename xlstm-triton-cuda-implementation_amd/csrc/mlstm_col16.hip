@@ -48,7 +48,7 @@ struct Col16Cfg {
 // phase B gathers 4 consecutive rows x 64 bytes (rows q and q+2 land in different halves of the row).
 __device__ __forceinline__ int gkey16(int q) { return (((q >> 1) & 1) << 2) | ((q >> 2) & 3); }
 
-template <typename T, int D>
+template <typename T, int D, bool DENSE>
 __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
     using R = Tr<T>;
@@ -110,16 +110,21 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
     const int kbA = wave >> 1, qbA = wave & 1;   // phase A block
     const int kbB = wave & 1, dsel = wave >> 1;  // phase B: keys 32*kbB.., column blocks dsel, dsel+2, ...
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN;
-    const T* Q = reinterpret_cast<const T*>(a.Q) + hoff * D;
-    const T* dH = reinterpret_cast<const T*>(a.dH) + hoff * D;
-    const T* K = reinterpret_cast<const T*>(a.K) + hoff * D;
-    const T* V = reinterpret_cast<const T*>(a.V) + hoff * D;
+    // the caller's tensors: q, k, v, dk, dv in layout la, dh in lb (element offset of the head, elements per position)
+    // (DENSE: contiguous [BH,S,D] tensors, strides as compile-time constants)
+    const size_t rsA = DENSE ? (size_t)D : (size_t)a.la.ss, rsB = DENSE ? (size_t)D : (size_t)a.lb.ss;
+    const size_t offA = DENSE ? hoff * D : a.la.head(bh), offB = DENSE ? hoff * D : a.lb.head(bh);
+    const T* Q = reinterpret_cast<const T*>(a.Q) + offA;
+    const T* dH = reinterpret_cast<const T*>(a.dH) + offB;
+    const T* K = reinterpret_cast<const T*>(a.K) + offA;
+    const T* V = reinterpret_cast<const T*>(a.V) + offA;
     const float* const beta_head = a.beta2 + poff;
     const float* const inv_head = a.inv_n + poff;
     const float* const db_head = a.db + poff;
 
     TileDma<T, D, GRAN, 256> tdma;
     tdma.init(tid);
+    const auto ra = tdma.rows(tid, (unsigned)(rsA * sizeof(T))), rb = tdma.rows(tid, (unsigned)(rsB * sizeof(T)));
     RowVec3Dma rvdma;   // beta, 1/n, db of a query tile (padded arrays: always readable)
     rvdma.init(tid, beta_head, inv_head, db_head);
     const int full_tiles = S / GRAN;  // query tiles whose 64 rows all exist
@@ -130,11 +135,11 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 #define COL_DMA(it, st)                                                          \
     do {                                                                         \
         if ((it) < full_tiles) {                                                 \
-            tdma.issue(ST_Q(st), Q + (size_t)GRAN * (it) * D);                    \
-            tdma.issue(ST_DH(st), dH + (size_t)GRAN * (it) * D);                  \
+            tdma.issue(ST_Q(st), Q + (size_t)GRAN * (it) * rsA, ra);              \
+            tdma.issue(ST_DH(st), dH + (size_t)GRAN * (it) * rsB, rb);            \
         } else {                                                                 \
-            tile_dma<T, D, GRAN, 256>(ST_Q(st), Q, GRAN * (it), S, tid);          \
-            tile_dma<T, D, GRAN, 256>(ST_DH(st), dH, GRAN * (it), S, tid);        \
+            tile_dma<T, D, GRAN, 256>(ST_Q(st), Q, GRAN * (it), S, tid, rsA);     \
+            tile_dma<T, D, GRAN, 256>(ST_DH(st), dH, GRAN * (it), S, tid, rsB);   \
         }                                                                        \
         rvdma.issue(ST_ROW(st), (it));                                            \
     } while (0)
@@ -150,11 +155,11 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
     constexpr int NTL = D / GRAN;   // 64-row tiles of a state
     const T* const Evc = has_state ? reinterpret_cast<const T*>(a.Ev) + ((size_t)bh * a.n_states + chunk) * D * D : nullptr;
     if (GRAN * (jt + 1) <= S) {
-        tdma.issue(Kt, K + (size_t)GRAN * jt * D);
-        tdma.issue(Vt, V + (size_t)GRAN * jt * D);
+        tdma.issue(Kt, K + (size_t)GRAN * jt * rsA, ra);
+        tdma.issue(Vt, V + (size_t)GRAN * jt * rsA, ra);
     } else {   // rows past the end are clamped
-        tile_dma<T, D, GRAN, 256>(Kt, K, GRAN * jt, S, tid);
-        tile_dma<T, D, GRAN, 256>(Vt, V, GRAN * jt, S, tid);
+        tile_dma<T, D, GRAN, 256>(Kt, K, GRAN * jt, S, tid, rsA);
+        tile_dma<T, D, GRAN, 256>(Vt, V, GRAN * jt, S, tid, rsA);
     }
     if (has_state) {
         tdma.issue(ST_Q(0), Evc);
@@ -297,8 +302,8 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
                     if (first_full) {
                         const int piece = (kb * NXW + x) * 4 + a4;
                         const int b0 = piece * 2 * PW0 / PIECES, b1 = (piece + 1) * 2 * PW0 / PIECES;   // of 2 PW0 blocks: Q then dH
-                        if (b0 < PW0) tdma.issue_range(ST_Q(0), Q + (size_t)GRAN * jt * D, b0, b1 < PW0 ? b1 : PW0);
-                        if (b1 > PW0) tdma.issue_range(ST_DH(0), dH + (size_t)GRAN * jt * D, b0 > PW0 ? b0 - PW0 : 0, b1 - PW0);
+                        if (b0 < PW0) tdma.issue_range(ST_Q(0), Q + (size_t)GRAN * jt * rsA, b0, b1 < PW0 ? b1 : PW0, ra);
+                        if (b1 > PW0) tdma.issue_range(ST_DH(0), dH + (size_t)GRAN * jt * rsB, b0 > PW0 ? b0 - PW0 : 0, b1 - PW0, rb);
                     }
                     const int d = 32 * (wave + XS * x) + 8 * a4 + 4 * h;
                     const f32x4 g4v = *reinterpret_cast<const f32x4*>(gv + d);
@@ -405,8 +410,8 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
                 if (it + 1 < NGe) { if (stage) COL_DMA(it + 1, 0); else COL_DMA(it + 1, 1); }
             }
         }
-        const T* gq = Q + (size_t)GRAN * (it + 1) * D;
-        const T* gdh = dH + (size_t)GRAN * (it + 1) * D;
+        const T* gq = Q + (size_t)GRAN * (it + 1) * rsA;
+        const T* gdh = dH + (size_t)GRAN * (it + 1) * rsB;
         T* const lq = ST_Q(stn);
         T* const ldh = ST_DH(stn);
         const T* Qs = ST_Q(stage);
@@ -493,7 +498,7 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             if constexpr (SPREAD && STAGES == 2) {
                 if (s % 4 == 0 && s / 4 < NH) {
                     const int k = idx * NH + s / 4;
-                    tdma.issue_range(lq, gq, k * PW / (4 * NH), (k + 1) * PW / (4 * NH));
+                    tdma.issue_range(lq, gq, k * PW / (4 * NH), (k + 1) * PW / (4 * NH), ra);
                 }
             }
         };
@@ -530,7 +535,7 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             if constexpr (SPREAD) {
                 if (idx < 2 && s % 4 == 2 && s / 4 < NH) {
                     const int k = idx * NH + s / 4;
-                    tdma.issue_range(ldh, gdh, k * PW / (4 * NH), (k + 1) * PW / (4 * NH));
+                    tdma.issue_range(ldh, gdh, k * PW / (4 * NH), (k + 1) * PW / (4 * NH), rb);
                 }
             }
         };
@@ -569,8 +574,8 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
             for (int r = 0; r < 8; r++) elem(1, r);
         } else {
             if constexpr (SPREAD) {   // (no MFMA chains to carry this wave's share of the next tile's copy)
-                tdma.issue(lq, gq);
-                tdma.issue_range(ldh, gdh, 0, PW / 2);
+                tdma.issue(lq, gq, ra);
+                tdma.issue_range(ldh, gdh, 0, PW / 2, rb);
             }
 #pragma unroll
             for (int x = 0; x < NXW; x++) read_qh(0, x);
@@ -606,7 +611,7 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
         for (int kb = 0; kb < NKB; kb++) read_gw(0, kb);
 #pragma unroll
         for (int t = 0; t < NQS; t++) {
-            if constexpr (SPREAD) { if (t < 2) tdma.issue_range(ldh, gdh, PW / 2 + t * PW / 4, PW / 2 + (t + 1) * PW / 4); }
+            if constexpr (SPREAD) { if (t < 2) tdma.issue_range(ldh, gdh, PW / 2 + t * PW / 4, PW / 2 + (t + 1) * PW / 4, rb); }
 #pragma unroll
             for (int x = 0; x < NXW; x++) {
 #pragma unroll
@@ -663,12 +668,12 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 #pragma unroll
         for (int which = 0; which < 2; which++) {
             const char* const stage = smem + which * Cfg::STAGE_BYTES;
-            char* const gout = reinterpret_cast<char*>(which ? a.dV : a.dK) + (hoff + (size_t)GRAN * jt) * D * sizeof(T);
+            char* const gout = reinterpret_cast<char*>(which ? a.dV : a.dK) + (offA + (size_t)GRAN * jt * rsA) * sizeof(T);
 #pragma unroll
             for (int i = 0; i < NPC; i++) {
                 const int c = tid + 256 * i, row = c / CPR, cc = c % CPR;
                 if (GRAN * jt + row < S) {
-                    *reinterpret_cast<uint4*>(gout + (size_t)row * D * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + row * RB + 16 * cc);
+                    *reinterpret_cast<uint4*>(gout + (size_t)row * rsA * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + row * RB + 16 * cc);
                 }
             }
         }
@@ -692,24 +697,25 @@ __global__ __launch_bounds__(256, 1) void col16_kernel(ColArgs a) {
 #endif
 }
 
-template <typename T, int D>
+template <typename T, int D, bool DENSE>
 static int launch_col16_t(const ColArgs& a, hipStream_t st) {
     using Cfg = Col16Cfg<T, D>;
-    auto kern = col16_kernel<T, D>;
-    if (hipError_t e = lds_limit_once<col16_kernel<T, D>>((int)(Cfg::LDS_BYTES + 2048 * sizeof(float))); e != hipSuccess) return (int)e;
+    auto kern = col16_kernel<T, D, DENSE>;
+    if (hipError_t e = lds_limit_once<col16_kernel<T, D, DENSE>>((int)(Cfg::LDS_BYTES + 2048 * sizeof(float))); e != hipSuccess) return (int)e;
     if (a.NG > 2048) return MLSTM_ESHAPE;
     hipLaunchKernelGGL(kern, dim3(a.BH * a.NG), dim3(256), Cfg::LDS_BYTES + (size_t)a.NG * sizeof(float), st, a);
     return (int)hipGetLastError();
 }
 
 int launch_col16_kernel(int dtype, int D, const ColArgs& a, hipStream_t st) {
+    const bool dense = is_dense(a.la, a.S, D) && is_dense(a.lb, a.S, D);
     if (D == 128) {
-        if (dtype == MLSTM_F16) return launch_col16_t<_Float16, 128>(a, st);
-        if (dtype == MLSTM_BF16) return launch_col16_t<__bf16, 128>(a, st);
+        if (dtype == MLSTM_F16) return dense ? launch_col16_t<_Float16, 128, true>(a, st) : launch_col16_t<_Float16, 128, false>(a, st);
+        if (dtype == MLSTM_BF16) return dense ? launch_col16_t<__bf16, 128, true>(a, st) : launch_col16_t<__bf16, 128, false>(a, st);
     }
     if (D == 256) {
-        if (dtype == MLSTM_F16) return launch_col16_t<_Float16, 256>(a, st);
-        if (dtype == MLSTM_BF16) return launch_col16_t<__bf16, 256>(a, st);
+        if (dtype == MLSTM_F16) return dense ? launch_col16_t<_Float16, 256, true>(a, st) : launch_col16_t<_Float16, 256, false>(a, st);
+        if (dtype == MLSTM_BF16) return dense ? launch_col16_t<__bf16, 256, true>(a, st) : launch_col16_t<__bf16, 256, false>(a, st);
     }
     return MLSTM_ESHAPE;
 }

@@ -245,8 +245,8 @@ __device__ __forceinline__ unsigned lds_offset_of(const void* p) {
 // Asynchronous copy of rows row0..row0+ROWS-1 of a [S, D] matrix into a swizzled tile.  `tile` must be the same for
 // all lanes of the wave.  Rows past S-1 are clamped (their products are masked or never stored).
 template <typename T, int D, int ROWS, int NT>
-__device__ __forceinline__ void tile_dma(T* tile, const T* g, int row0, int S, int tid) {
-    using Z = Swz<T, D>;
+__device__ __forceinline__ void tile_dma(T* tile, const T* g, int row0, int S, int tid, size_t row_stride = D) {
+    using Z = Swz<T, D>;   // (row_stride: elements between the matrix' rows in memory)
     constexpr int NW = NT / 64, BLOCKS = ROWS * Z::CPR / 64;
     static_assert(BLOCKS % NW == 0, "tile must divide evenly over the waves");
     const int wave = tid >> 6, lane = tid & 63;
@@ -259,7 +259,7 @@ __device__ __forceinline__ void tile_dma(T* tile, const T* g, int row0, int S, i
         const int c = pc ^ Z::key(r);
         int gr = row0 + r;
         gr = gr < S ? gr : S - 1;
-        dma16(g + (size_t)gr * D + c * Z::EPC, __builtin_amdgcn_readfirstlane(base + blk * 1024));
+        dma16(g + (size_t)gr * row_stride + c * Z::EPC, __builtin_amdgcn_readfirstlane(base + blk * 1024));
     }
 }
 
@@ -327,6 +327,34 @@ struct TileDma {
         for (int it = 0; it < PER_WAVE; it++)
             dma16_s(reinterpret_cast<const char*>(g_tile) + (it / PERIOD) * GROUP_BYTES, voff[it % PERIOD], base, (it * NW + wave_s) * 1024);
     }
+    // The same copies from a matrix whose rows lie `row_bytes` apart in memory (a tensor of the caller's in a layout of
+    // its own; init's offsets serve matrices with D elements per row, such as the chunk states).  rows() after init().
+    struct Rows { unsigned voff[PERIOD]; unsigned group_bytes; };
+    __device__ __forceinline__ Rows rows(int tid, unsigned row_bytes) const {
+        Rows o;
+        const int lane = tid & 63;
+#pragma unroll
+        for (int it = 0; it < PERIOD; it++) {
+            const int p = (it * NW + wave_s) * 64 + lane;
+            const int r = p / Z::CPR, pc = p % Z::CPR;
+            o.voff[it] = (unsigned)r * row_bytes + (unsigned)((pc ^ Z::key(r)) << 4);
+        }
+        o.group_bytes = (unsigned)(PERIOD * RSTEP) * row_bytes;
+        return o;
+    }
+    __device__ __forceinline__ void issue_range(T* tile, const T* g_tile_v, int first, int last, const Rows& o) const {
+        const unsigned base = __builtin_amdgcn_readfirstlane(lds_offset_of(tile));
+        const unsigned long long gv = (unsigned long long)(size_t)g_tile_v;
+        const unsigned long long gs = ((unsigned long long)(unsigned)__builtin_amdgcn_readfirstlane((int)(gv >> 32)) << 32) |
+                                      (unsigned)__builtin_amdgcn_readfirstlane((int)gv);
+        const void* g_tile = (const void*)(size_t)gs;
+        const unsigned gb = __builtin_amdgcn_readfirstlane(o.group_bytes);
+#pragma unroll
+        for (int it = 0; it < PER_WAVE; it++)
+            if (it >= first && it < last)
+                dma16_s(reinterpret_cast<const char*>(g_tile) + (size_t)((it / PERIOD) * gb), o.voff[it % PERIOD], base, (it * NW + wave_s) * 1024);
+    }
+    __device__ __forceinline__ void issue(T* tile, const T* g_tile_v, const Rows& o) const { issue_range(tile, g_tile_v, 0, PER_WAVE, o); }
 };
 
 // 64 floats (one per key of a tile) by the first wave

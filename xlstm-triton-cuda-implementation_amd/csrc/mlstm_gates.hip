@@ -71,31 +71,42 @@ __device__ __forceinline__ void gates_outputs(float c, float al, bool ok, double
     if (lane == 0) G2[gidx] = Gg * LOG2E_D;
 }
 
+// log-sigmoid of the forget gate at position t from what the caller's F holds (see launch_gates): the pre-activation,
+// the log-sigmoid itself, or its cumulative sum over the head (then the difference of two neighbours)
+template <typename TG>
+__device__ __forceinline__ float forget_log(const TG* f, size_t ss, int t, int form) {
+    const float x = (float)f[(size_t)t * ss];
+    if (form == MLSTM_GATE_RAW) return log_sigmoid(x);
+    if (form == MLSTM_GATE_LOGSIGMOID) return x;
+    return t > 0 ? x - (float)f[(size_t)(t - 1) * ss] : x;
+}
+
 // Sequences of up to 16 * GPW granules: every wave keeps its granules' cumulative sums and alphas in registers
 // between the two passes, and issues all its loads before the first scan (one memory round trip instead of one per granule
 // and pass).
 template <typename TG, int GPW>
 __global__ __launch_bounds__(1024) void gates_kernel_reg(const TG* __restrict__ F, const TG* __restrict__ I, float* __restrict__ alpha2,
                                                         float* __restrict__ beta2, double* __restrict__ G2, float* __restrict__ M,
-                                                        float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG) {
+                                                        float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form) {
     __shared__ double sT[16 * GPW];
     __shared__ double sP[16 * GPW];
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const TG* f = F + (size_t)bh * S;
-    const TG* ig = I + (size_t)bh * S;
+    const size_t gs = (size_t)lg.ss;
+    const TG* f = F + lg.head(bh);
+    const TG* ig = I + lg.head(bh);
     float fv[GPW], iv[GPW], c[GPW], al[GPW];
 #pragma unroll
     for (int k = 0; k < GPW; k++) {
         const int t = (wave + 16 * k) * GRAN + lane;
         const bool ok = t < S;
-        fv[k] = ok ? (float)f[t] : 0.0f;
-        iv[k] = ok ? (float)ig[t] : 0.0f;
+        fv[k] = ok ? forget_log(f, gs, t, form) : 0.0f;
+        iv[k] = ok ? (float)ig[(size_t)t * gs] : 0.0f;
     }
 #pragma unroll
     for (int k = 0; k < GPW; k++) {
         const int g = wave + 16 * k, t = g * GRAN + lane;
         const bool ok = t < S;
-        const float lf = ok ? log_sigmoid(fv[k]) : 0.0f;
+        const float lf = ok ? fv[k] : 0.0f;
         c[k] = wave_scan_inclusive<OpAdd>(lf);
         al[k] = ok ? iv[k] - c[k] : -INFINITY;
         const float p = wave_reduce<OpMax>(al[k]);
@@ -117,20 +128,21 @@ __global__ __launch_bounds__(1024) void gates_kernel_reg(const TG* __restrict__ 
 template <typename TG>
 __global__ __launch_bounds__(1024) void gates_kernel(const TG* __restrict__ F, const TG* __restrict__ I, float* __restrict__ alpha2,
                                                     float* __restrict__ beta2, double* __restrict__ G2, float* __restrict__ M,
-                                                    float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG) {
+                                                    float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form) {
     __shared__ double sT[GATES_MAX_GRANULES];  // granule totals of lf, then exclusive prefix G
     __shared__ double sP[GATES_MAX_GRANULES];  // granule maxima of alpha, then running max R of (P - G) over earlier granules
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const TG* f = F + (size_t)bh * S;
-    const TG* ig = I + (size_t)bh * S;
+    const size_t gs = (size_t)lg.ss;
+    const TG* f = F + lg.head(bh);
+    const TG* ig = I + lg.head(bh);
 
     // pass 1: per-granule total of lf and maximum of alpha
     for (int g = wave; g < NG; g += 16) {
         int t = g * GRAN + lane;
         bool ok = t < S;
-        float lf = ok ? log_sigmoid((float)f[t]) : 0.0f;
+        float lf = ok ? forget_log(f, gs, t, form) : 0.0f;
         float c = wave_scan_inclusive<OpAdd>(lf);
-        float al = ok ? (float)ig[t] - c : -INFINITY;
+        float al = ok ? (float)ig[(size_t)t * gs] - c : -INFINITY;
         float p = wave_reduce<OpMax>(al);
         float tot = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, c), 63));
         if (lane == 0) { sT[g] = (double)tot; sP[g] = (double)p; }
@@ -142,9 +154,9 @@ __global__ __launch_bounds__(1024) void gates_kernel(const TG* __restrict__ F, c
     for (int g = wave; g < NG; g += 16) {
         int t = g * GRAN + lane;
         bool ok = t < S;
-        float lf = ok ? log_sigmoid((float)f[t]) : 0.0f;
+        float lf = ok ? forget_log(f, gs, t, form) : 0.0f;
         float c = wave_scan_inclusive<OpAdd>(lf);
-        float al = ok ? (float)ig[t] - c : -INFINITY;
+        float al = ok ? (float)ig[(size_t)t * gs] - c : -INFINITY;
         gates_outputs(c, al, ok, sT[g], sP[g], (size_t)bh * NG * GRAN + t, (size_t)bh * S + t, (size_t)bh * NG + g, lane, alpha2, beta2, G2, M,
                       ek2, amax2);
     }
@@ -152,24 +164,25 @@ __global__ __launch_bounds__(1024) void gates_kernel(const TG* __restrict__ F, c
 
 template <typename TG>
 static hipError_t launch_gates_t(const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                                 float* amax2, int BH, int S, hipStream_t st) {
+                                 float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form) {
     int NG = (S + GRAN - 1) / GRAN;
     if (NG <= 16 * 4)
-        hipLaunchKernelGGL((gates_kernel_reg<TG, 4>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG);
+        hipLaunchKernelGGL((gates_kernel_reg<TG, 4>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
     else if (NG <= 16 * 8)
-        hipLaunchKernelGGL((gates_kernel_reg<TG, 8>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG);
+        hipLaunchKernelGGL((gates_kernel_reg<TG, 8>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
     else
-        hipLaunchKernelGGL(gates_kernel<TG>, dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG);
+        hipLaunchKernelGGL(gates_kernel<TG>, dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
     return hipGetLastError();
 }
 
 hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                        float* amax2, int BH, int S, hipStream_t st) {
+                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form) {
     if ((S + GRAN - 1) / GRAN > GATES_MAX_GRANULES) return hipErrorInvalidValue;
+    if (form == MLSTM_GATE_CUMSUM && gate_dtype != MLSTM_F32) return hipErrorInvalidValue;   // (16-bit types cannot hold the sum)
     switch (gate_dtype) {
-        case MLSTM_F32: return launch_gates_t<float>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st);
-        case MLSTM_F16: return launch_gates_t<_Float16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st);
-        case MLSTM_BF16: return launch_gates_t<__bf16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st);
+        case MLSTM_F32: return launch_gates_t<float>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
+        case MLSTM_F16: return launch_gates_t<_Float16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
+        case MLSTM_BF16: return launch_gates_t<__bf16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
     }
     return hipErrorInvalidValue;
 }

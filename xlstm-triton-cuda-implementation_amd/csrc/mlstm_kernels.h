@@ -17,10 +17,29 @@ inline hipError_t lds_limit_once(int bytes) {
 }
 constexpr int GATE_GRANULE = 64;  // positions per gate granule (== mlstm::GRAN in the device code)
 
+// Where a [B,NH,S,D] (or [B,NH,S]) tensor of the caller's keeps position s of head bh = b * NH + h: at element
+// b * sb + h * sh + s * ss (+ the column: the last dimension is contiguous).  Everything the library owns (workspace,
+// statistics m and b, chunk states) is dense.
+struct Lay {
+    long long sb, sh, ss;
+    int NH;
+    __host__ __device__ size_t head(int bh) const { return (size_t)((long long)(bh / NH) * sb + (long long)(bh % NH) * sh); }
+};
+inline Lay dense_layout(int NH, long long S, long long D) { return Lay{(long long)NH * S * D, S * D, D, NH}; }
+// dense [B,NH,S,D]?  (The tile kernels keep a variant with the strides as compile-time constants for that case: run-time
+// strides cost them address arithmetic in loops that are bound by instruction issue.)
+inline bool is_dense(const Lay& l, long long S, long long D) { return l.ss == D && l.sh == S * D && l.sb == (long long)l.NH * S * D; }
+
 // Gate pre-pass: alpha2, beta2 [BH, NG*64] fp32 (NG = ceil(S/64), rows padded), G2 [BH, NG] fp64, M [BH,S] fp32.
 // ek2 [BH, NG*64] = exp2(alpha2 - block max), amax2 [BH, NG*2] = the maxima of alpha2 over blocks of 32 positions.
+// lg: layout of F and I.  gate_form: what F holds (MLSTM_GATE_RAW: the forget gate's pre-activation, _LOGSIGMOID: its
+// log-sigmoid, _CUMSUM: the cumulative sum of that over the positions of a head).
 hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                        float* amax2, int BH, int S, hipStream_t st);
+                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int gate_form);
+inline hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
+                               float* amax2, int BH, int S, hipStream_t st) {
+    return launch_gates(gate_dtype, F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, dense_layout(BH, S, 1), MLSTM_GATE_RAW);
+}
 
 extern bool g_force_generic;  // see mlstm_force_generic_kernels
 
@@ -67,6 +86,9 @@ struct RowArgs {
     // see mlstm_kernel_error) and the kernel runs on to its end.  spin_limit < 0 (test aid) lets every wait expire.
     int* err;
     int spin_limit;
+    // layouts of the caller's tensors: la for q, k, v (forward: X, Y1, Y2; dQ pass: Y1, Y2, Qrow and out),
+    // lb for h, dh, o (forward: out, O, out_gated; dQ pass: X), lh for Hin (the caller's h, or a dense recomputed one)
+    Lay la, lb, lh;
 };
 // mode 0 = forward (H, b), mode 1 = dQ
 int launch_row_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);
@@ -98,6 +120,7 @@ struct ColArgs {
     const void* Ev;          // [BH][n_states][D][D] reverse states, value-major (ChunkArgs::CstT of the reverse pass)
     const float* gvec;       // [BH][n_states][D]
     int precise;             // split mode (see RowArgs): G and W enter phase B as hi + lo
+    Lay la, lb;              // layouts of Q, K, V, dK, dV (la) and of dH (lb)
 };
 int launch_col_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
 // phase A as 16x16x32 products on two query halves, the element-wise part of the first between the MFMAs of the second;
@@ -121,6 +144,8 @@ struct DfArgs {
     const float* rowinter;
     const float* anchor;     // [BH][n_states]: the running sum of (col - row) at the first position of chunks 1, 2, ...
     int n_states;
+    Lay lg;                  // layout of F, dF and dI
+    int gate_form;           // what F holds (see launch_gates); dF is the gradient of that same quantity
 };
 int launch_df(int gate_dtype, const DfArgs& a, hipStream_t st);
 
@@ -143,6 +168,7 @@ struct ChunkArgs {
     int reverse;
     const float* inv_n;
     const float* db;
+    Lay lk, lv;           // layouts of K and V
 };
 int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st);
 

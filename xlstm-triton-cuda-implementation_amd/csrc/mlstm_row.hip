@@ -65,13 +65,17 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     const int row = r0 + c32, rowc = row < S ? row : S - 1;
     const bool wave_active = r0 < S;
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN;
-    const T* X = reinterpret_cast<const T*>(a.X) + hoff * D;
-    const T* Y1 = reinterpret_cast<const T*>(a.Y1) + hoff * D;
-    const T* Y2 = reinterpret_cast<const T*>(a.Y2) + hoff * D;
+    // the caller's tensors: q, k, v, dq in layout la, h, dh, o in lb (element offset of the head, elements per position)
+    const size_t rsA = (size_t)a.la.ss, rsB = (size_t)a.lb.ss, offA = a.la.head(bh), offB = a.lb.head(bh);
+    const size_t rsX = MODE == MODE_FWD ? rsA : rsB, offX = MODE == MODE_FWD ? offA : offB;
+    const size_t rsO = MODE == MODE_FWD ? rsB : rsA, offO = MODE == MODE_FWD ? offB : offA;
+    const T* X = reinterpret_cast<const T*>(a.X) + offX;
+    const T* Y1 = reinterpret_cast<const T*>(a.Y1) + offA;
+    const T* Y2 = reinterpret_cast<const T*>(a.Y2) + offA;
 
     frag xf[NS];
 #pragma unroll
-    for (int s = 0; s < NS; s++) xf[s] = frag_rowmajor<T>(X + (size_t)rowc * D, s, h);
+    for (int s = 0; s < NS; s++) xf[s] = frag_rowmajor<T>(X + (size_t)rowc * rsX, s, h);
 
     // granule bases of this head in LDS: a global load inside the main loop would have to be waited for with
     // vmcnt(0), which would also wait for the tile copies in flight
@@ -82,7 +86,7 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     if constexpr (MODE == MODE_DQ) {
         const T* hlo = nullptr;
         if constexpr (STRICT) { if (a.Hin_lo) hlo = reinterpret_cast<const T*>(a.Hin_lo) + (hoff + rowc) * D; }
-        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + (hoff + rowc) * D, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv, hlo);
+        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + a.lh.head(bh) + (size_t)rowc * (size_t)a.lh.ss, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv, hlo);
         if (row < S && h == 0) { a.inv_n[poff + row] = inv_n; a.db[poff + row] = dbv; }
     }
 #pragma unroll
@@ -113,17 +117,18 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     const float* const amax_head = a.amax2 + (size_t)bh * NG * 2;
     TileDma<T, D, GRAN, 256> tdma;
     tdma.init(tid);
+    const auto ra = tdma.rows(tid, (unsigned)(rsA * sizeof(T)));
     RowVec3Dma rvdma;   // alpha, ek (64 per tile) and the two block maxima of a tile (padded arrays: always readable)
     rvdma.init(tid, alpha_head, ek_head, amax_head, 64, 64, 2);
     const int full_tiles = S / GRAN;  // key tiles whose 64 rows all exist
 #define ROW_DMA(j, st)                                                                   \
     do {                                                                                 \
         if ((j) < full_tiles) {                                                          \
-            tdma.issue(ST_Y1(st), Y1 + (size_t)GRAN * (j) * D);                           \
-            tdma.issue(ST_Y2(st), Y2 + (size_t)GRAN * (j) * D);                           \
+            tdma.issue(ST_Y1(st), Y1 + (size_t)GRAN * (j) * rsA, ra);                     \
+            tdma.issue(ST_Y2(st), Y2 + (size_t)GRAN * (j) * rsA, ra);                     \
         } else {                                                                         \
-            tile_dma<T, D, GRAN, 256>(ST_Y1(st), Y1, GRAN * (j), S, tid);                 \
-            tile_dma<T, D, GRAN, 256>(ST_Y2(st), Y2, GRAN * (j), S, tid);                 \
+            tile_dma<T, D, GRAN, 256>(ST_Y1(st), Y1, GRAN * (j), S, tid, rsA);            \
+            tile_dma<T, D, GRAN, 256>(ST_Y2(st), Y2, GRAN * (j), S, tid, rsA);            \
         }                                                                                \
         rvdma.issue(ST_AL(st), (j));                                                     \
     } while (0)
@@ -328,12 +333,12 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
         __syncthreads();  // tile j has landed for every wave and stage (j+1)&1 is free again
         const int jn = j + 1, stn = jn & 1;
         rvdma.issue(ST_AL(stn), jn);
-        const T* gy1 = Y1 + (size_t)GRAN * jn * D;
-        const T* gy2 = Y2 + (size_t)GRAN * jn * D;
+        const T* gy1 = Y1 + (size_t)GRAN * jn * rsA;
+        const T* gy2 = Y2 + (size_t)GRAN * jn * rsA;
         T* const ly1 = ST_Y1(stn);
         T* const ly2 = ST_Y2(stn);
-        auto hook1 = [&](int idx, int n) { tdma.issue_range(ly1, gy1, idx * PW / n, (idx + 1) * PW / n); };
-        auto hook2 = [&](int idx, int n) { tdma.issue_range(ly2, gy2, idx * PW / n, (idx + 1) * PW / n); };
+        auto hook1 = [&](int idx, int n) { tdma.issue_range(ly1, gy1, idx * PW / n, (idx + 1) * PW / n, ra); };
+        auto hook2 = [&](int idx, int n) { tdma.issue_range(ly2, gy2, idx * PW / n, (idx + 1) * PW / n, ra); };
         const T* y1 = ST_Y1(j & 1);
         const T* y2 = ST_Y2(j & 1);
         const float* sal = ST_AL(j & 1);
@@ -405,7 +410,7 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
         if (row < S && h == 0) a.Bsum[hoff + row] = b;
     }
     if (row < S) {
-        T* out = reinterpret_cast<T*>(a.out) + (hoff + row) * D;
+        T* out = reinterpret_cast<T*>(a.out) + offO + (size_t)row * rsO;
 #pragma unroll
         for (int d = 0; d < NDB; d++)
 #pragma unroll
@@ -424,8 +429,8 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
             }
         if constexpr (MODE == MODE_FWD) {
             if (a.O) {  // gated copy from the fp32 accumulators
-                const T* og = reinterpret_cast<const T*>(a.O) + (hoff + row) * D;
-                T* outg = reinterpret_cast<T*>(a.out_gated) + (hoff + row) * D;
+                const T* og = reinterpret_cast<const T*>(a.O) + offB + (size_t)row * rsB;
+                T* outg = reinterpret_cast<T*>(a.out_gated) + offB + (size_t)row * rsB;
 #pragma unroll
                 for (int d = 0; d < NDB; d++)
 #pragma unroll

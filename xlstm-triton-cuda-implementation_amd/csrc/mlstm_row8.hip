@@ -36,7 +36,7 @@ struct Row8Cfg {
     static constexpr size_t FIXED_BYTES = 4 * TILE_BYTES + 2 * AUX_BYTES + PBUF_BYTES + MISC_BYTES;  // + NG doubles
 };
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool DENSE>
 __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using R = Tr<T>;
@@ -93,6 +93,14 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         }
     }
     size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN, goff = (size_t)bh * NG;
+    // The caller's tensors: q, k, v, dq in one layout (la), h, dh, o in another (lb); offA / offB: element offset of the
+    // head's first position, rsA / rsB: elements from one position to the next.  X and the output change sides between
+    // the forward (Q -> H) and the dQ pass (dH -> dQ).
+    // (DENSE: every tensor is a contiguous [BH,S,D]; the strides are then compile-time constants)
+    const size_t rsA = DENSE ? (size_t)D : (size_t)a.la.ss, rsB = DENSE ? (size_t)D : (size_t)a.lb.ss;
+    size_t offA = DENSE ? hoff * D : a.la.head(bh), offB = DENSE ? hoff * D : a.lb.head(bh);
+    size_t rsH = DENSE ? (size_t)D : 0, offH = DENSE ? hoff * D : 0;   // Hin (dQ pass)
+    if constexpr (MODE == R8_DQ && !DENSE) { rsH = (size_t)a.lh.ss; offH = a.lh.head(bh); }
     // Long sequences in chunks: the workgroup's rows lie in chunk `chunk` of chunk_len positions.  Everything below addresses
     // positions relative to the chunk's first one (the sequence "starts" there: per-position offsets move forward, S, NG
     // and the row tile index shrink); what lies before the chunk enters through the state of the previous chunk.
@@ -101,6 +109,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         chunk = (qt * R8_BQ) / a.chunk_len;
         const int p0 = chunk * a.chunk_len;
         hoff += p0; poff += p0; goff += p0 / GRAN;
+        offA += (size_t)p0 * rsA; offB += (size_t)p0 * rsB; offH += (size_t)p0 * rsH;
         S -= p0; NG -= p0 / GRAN; qt -= p0 / R8_BQ;
     }
     const int q0 = qt * R8_BQ, r0 = q0 + 64 * rg;            // r0: first of the wave's 64 rows (a multiple of 64)
@@ -108,8 +117,10 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
     int rowc[2];
 #pragma unroll
     for (int r = 0; r < 2; r++) { const int row = r0 + 32 * r + c32; rowc[r] = row < S ? row : S - 1; }
-    const T* Y1 = reinterpret_cast<const T*>(a.Y1) + hoff * D;
-    const T* Y2 = reinterpret_cast<const T*>(a.Y2) + hoff * D;
+    const size_t rsX = MODE == R8_FWD ? rsA : rsB, offX = MODE == R8_FWD ? offA : offB;
+    const size_t rsO = MODE == R8_FWD ? rsB : rsA, offO = MODE == R8_FWD ? offB : offA;
+    const T* Y1 = reinterpret_cast<const T*>(a.Y1) + offA;
+    const T* Y2 = reinterpret_cast<const T*>(a.Y2) + offA;
     const int last_row = (q0 + R8_BQ - 1 < S - 1) ? q0 + R8_BQ - 1 : S - 1;
     const int nJ = last_row / GRAN + 1;
     const int full_tiles = S / GRAN;
@@ -129,24 +140,25 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
 
     TileDma<T, D, GRAN, 256> tdma;
     tdma.init(rtid);
+    const auto ra = tdma.rows(rtid, (unsigned)(rsA * sizeof(T)));   // Y1, Y2 tiles
     constexpr int PW = TileDma<T, D, GRAN, 256>::PER_WAVE;
     frag* const p_rg = pbuf + rg * (2 * 4 * 64) + lane;        // fragment (r, g) of the row group -> p_rg[(4*r + g) * 64]
 
     if (producer) {
         // ------------------------------------------------------------------------------------------ producers
         const int kh = sub;
-        const T* X = reinterpret_cast<const T*>(a.X) + hoff * D;
+        const T* X = reinterpret_cast<const T*>(a.X) + offX;
         {   // first of all the copy of the first Y1 tile: its latency then overlaps that of the plain loads below
             T* dst = reinterpret_cast<T*>(y1s);
-            if (0 < full_tiles) tdma.issue(dst, Y1);
-            else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid);
+            if (0 < full_tiles) tdma.issue(dst, Y1, ra);
+            else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
         }
         frag xf[2][NS];
         float crow_base[2], inv_n[2] = {0.f, 0.f}, dbv[2] = {0.f, 0.f}, bsum[2] = {0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < 2; r++) {
 #pragma unroll
-            for (int s = 0; s < NS; s++) xf[r][s] = frag_rowmajor<T>(X + (size_t)rowc[r] * D, s, h);
+            for (int s = 0; s < NS; s++) xf[r][s] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, s, h);
             crow_base[r] = -0.5f * __log2f((float)D) - a.beta2[poff + rowc[r]];
         }
         if constexpr (MODE == R8_DQ) {
@@ -157,7 +169,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             if (chunk > 0) {
                 float inv = 0.f, dbr = 0.f;
                 const int rc = rowc[kh];
-                const T* hrow = reinterpret_cast<const T*>(a.Hin) + (hoff + rc) * D;
+                const T* hrow = reinterpret_cast<const T*>(a.Hin) + offH + (size_t)rc * rsH;
                 if (kh == 0) row_stats<T, NS>(xf[0], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
                 else row_stats<T, NS>(xf[1], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
                 const int row = r0 + 32 * kh + c32;
@@ -184,8 +196,8 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         auto aux_dma = [&](int j) { rvdma.issue(auxs + (j & 1) * 3 * GRAN, j); };
         auto y1_bulk = [&](int j) {
             T* dst = reinterpret_cast<T*>(y1s + (j & 1) * Cfg::TILE_BYTES);
-            if (j < full_tiles) tdma.issue(dst, Y1 + (size_t)GRAN * j * D);
-            else tile_dma<T, D, GRAN, 256>(dst, Y1, GRAN * j, S, rtid);
+            if (j < full_tiles) tdma.issue(dst, Y1 + (size_t)GRAN * j * rsA, ra);
+            else tile_dma<T, D, GRAN, 256>(dst, Y1, GRAN * j, S, rtid, rsA);
             aux_dma(j);
         };
         // s_r = (32 keys of this wave) x (row block r); every Y1 fragment feeds both row blocks.  The operand reads run
@@ -321,8 +333,8 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         int j = 0;
         if (jspread > 0) {
             T* const ly1 = reinterpret_cast<T*>(y1s + Cfg::TILE_BYTES);
-            const T* gy1 = Y1 + (size_t)GRAN * D;
-            main_tile(0, [&](int idx, int n) { tdma.issue_range(ly1, gy1, idx * PW / n, (idx + 1) * PW / n); });
+            const T* gy1 = Y1 + (size_t)GRAN * rsA;
+            main_tile(0, [&](int idx, int n) { tdma.issue_range(ly1, gy1, idx * PW / n, (idx + 1) * PW / n, ra); });
             j = 1;
         }
         for (; j < jspread; j++) main_tile(j, no_hook);
@@ -380,11 +392,11 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         uint4 og[CPR];
         if constexpr (MODE == R8_FWD) {
             if (a.O) {
-                const char* const go = reinterpret_cast<const char*>(a.O) + ((hoff + r0) * D + (size_t)kh * (D / 2)) * sizeof(T);
+                const char* const go = reinterpret_cast<const char*>(a.O) + (offB + (size_t)r0 * rsB + (size_t)kh * (D / 2)) * sizeof(T);
 #pragma unroll
                 for (int x = 0; x < CPR; x++) {
                     const int c = lane + 64 * x, rr = c / CPR, cc = c % CPR;
-                    og[x] = r0 + rr < S ? *reinterpret_cast<const uint4*>(go + (size_t)rr * D * sizeof(T) + 16 * cc) : uint4{0, 0, 0, 0};
+                    og[x] = r0 + rr < S ? *reinterpret_cast<const uint4*>(go + (size_t)rr * rsB * sizeof(T) + 16 * cc) : uint4{0, 0, 0, 0};
                 }
             }
         }
@@ -403,7 +415,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 typedef typename R::vec4 V4;
                 struct Pair { V4 lo, hi; };
                 const char* const stage = smem + wave * 64 * RB;
-                char* const gg = reinterpret_cast<char*>(a.out_gated) + ((hoff + r0) * D + (size_t)kh * (D / 2)) * sizeof(T);
+                char* const gg = reinterpret_cast<char*>(a.out_gated) + (offB + (size_t)r0 * rsB + (size_t)kh * (D / 2)) * sizeof(T);
 #pragma unroll
                 for (int x = 0; x < CPR; x++) {
                     const int c = lane + 64 * x, rr = c / CPR, cc = c % CPR;
@@ -412,7 +424,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                     Pair res;
                     res.lo = gate4<T>(hv.lo, ov.lo);
                     res.hi = gate4<T>(hv.hi, ov.hi);
-                    if (r0 + rr < S) *reinterpret_cast<Pair*>(gg + (size_t)rr * D * sizeof(T) + 16 * cc) = res;
+                    if (r0 + rr < S) *reinterpret_cast<Pair*>(gg + (size_t)rr * rsB * sizeof(T) + 16 * cc) = res;
                 }
             }
         }
@@ -430,8 +442,8 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         vrd.init(lane, NDH * dh);
         auto y2_bulk = [&](int j) {
             T* dst = reinterpret_cast<T*>(y2s + (j & 1) * Cfg::TILE_BYTES);
-            if (j < full_tiles) tdma.issue(dst, Y2 + (size_t)GRAN * j * D);
-            else tile_dma<T, D, GRAN, 256>(dst, Y2, GRAN * j, S, rtid);
+            if (j < full_tiles) tdma.issue(dst, Y2 + (size_t)GRAN * j * rsA, ra);
+            else tile_dma<T, D, GRAN, 256>(dst, Y2, GRAN * j, S, rtid, rsA);
         };
         // fragments of one tile into registers, then tell the producers their buffer is free again
         auto take = [&](frag (&pf)[2][4]) {
@@ -485,14 +497,14 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         // only "used" behind the state tiles: a use here would wait for them, and for every copy issued before them.
         int touched[2] = {0, 0};
         if (MODE == R8_DQ && chunk > 0) {
-            const char* qb = reinterpret_cast<const char*>(a.Qrow) + (hoff * D + (size_t)dh * (D / 2)) * sizeof(T);
+            const char* qb = reinterpret_cast<const char*>(a.Qrow) + (offA + (size_t)dh * (D / 2)) * sizeof(T);
             constexpr int LINES = (D / 2) * (int)sizeof(T) / 128;   // 128-byte lines of this wave's half of a row
 #pragma unroll
             for (int r = 0; r < 2; r++) {
 #pragma unroll
                 for (int ln = 0; ln < LINES; ln += 2) {
                     if (ln + h < LINES)   // (the two lanes of a row take a line each; never past the end of the half row)
-                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * D * sizeof(T) + 128 * (ln + h));
+                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * rsA * sizeof(T) + 128 * (ln + h));
                 }
             }
         }
@@ -500,13 +512,13 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             // Per-row scalars of the backward for row block r = dh of the row group (the producers need them from their
             // first tile on, the column kernel reads them from global memory): this role idles until the first P arrives.
             // (Behind the first chunk the producers compute them: see there.)
-            const T* X = reinterpret_cast<const T*>(a.X) + hoff * D;
+            const T* X = reinterpret_cast<const T*>(a.X) + offX;
             const int rc = rowc[dh];
             frag xs[NS];
 #pragma unroll
-            for (int s = 0; s < NS; s++) xs[s] = frag_rowmajor<T>(X + (size_t)rc * D, s, h);
+            for (int s = 0; s < NS; s++) xs[s] = frag_rowmajor<T>(X + (size_t)rc * rsX, s, h);
             float inv = 0.f, dbr = 0.f;
-            row_stats<T, NS>(xs, reinterpret_cast<const T*>(a.Hin) + (hoff + rc) * D, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
+            row_stats<T, NS>(xs, reinterpret_cast<const T*>(a.Hin) + offH + (size_t)rc * rsH, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
             const int row = r0 + 32 * dh + c32;
             if (h == 0) {
                 *reinterpret_cast<float2*>(bex + ((rg * 2 + dh) * 32 + c32) * 2) = make_float2(inv, dbr);
@@ -522,7 +534,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             // from global memory: the state's rows are stored in the order in which this product contracts them.
             //   forward: H^T += C~^T-tiles x Q^T, then the rows' decay exp(A_e - A_i)
             //   dQ pass: dQ^T += C~-tiles x dH^T, then decay / n; and the rank-one term decay * db_i * n~
-            const T* X = reinterpret_cast<const T*>(a.X) + hoff * D;
+            const T* X = reinterpret_cast<const T*>(a.X) + offX;
             auto none = [](int, int) {};
 #pragma unroll 1
             for (int pp = 0; pp < D / 64; pp += 2) {
@@ -535,8 +547,8 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 for (int r = 0; r < 2; r++)
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        pf0[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * D, 4 * pp + g, h);
-                        pf1[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * D, 4 * pp + 4 + g, h);
+                        pf0[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, 4 * pp + g, h);
+                        pf1[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, 4 * pp + 4 + g, h);
                     }
                 dma_wait();
                 __syncthreads();
@@ -568,7 +580,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 asm volatile("" ::"v"(touched[0]), "v"(touched[1]));
                 // Row sums of dD over the keys before the chunk: q_i . dQ_i of what the accumulators hold now; this wave's
                 // half of the columns goes to LDS, the halves meet behind the next barrier
-                const T* Qh = reinterpret_cast<const T*>(a.Qrow) + hoff * D + (size_t)dh * (D / 2);
+                const T* Qh = reinterpret_cast<const T*>(a.Qrow) + offA + (size_t)dh * (D / 2);
 #pragma unroll
                 for (int r = 0; r < 2; r++) {
                     float rp = 0.f;
@@ -577,7 +589,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
 #pragma unroll
                         for (int a4 = 0; a4 < 4; a4++) {
                             const f32x4 qv = __builtin_convertvector(
-                                *reinterpret_cast<const typename R::vec4*>(Qh + (size_t)rowc[r] * D + 32 * d + 8 * a4 + 4 * h), f32x4);
+                                *reinterpret_cast<const typename R::vec4*>(Qh + (size_t)rowc[r] * rsA + 32 * d + 8 * a4 + 4 * h), f32x4);
 #pragma unroll
                             for (int c = 0; c < 4; c++) rp += oacc[r][d][4 * a4 + c] * qv[c];
                         }
@@ -612,10 +624,10 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             frag pf[2][4];
             take(pf);
             if constexpr (decltype(copy_y1_tag)::value)
-                tdma.issue(reinterpret_cast<T*>(y1s + ((i + 1) & 1) * Cfg::TILE_BYTES), Y1 + (size_t)GRAN * (i + 1) * D);
+                tdma.issue(reinterpret_cast<T*>(y1s + ((i + 1) & 1) * Cfg::TILE_BYTES), Y1 + (size_t)GRAN * (i + 1) * rsA, ra);
             T* const ly2 = reinterpret_cast<T*>(y2s + (i & 1) * Cfg::TILE_BYTES);
-            const T* gy2 = Y2 + (size_t)GRAN * i * D;
-            auto hook = [&](int idx, int n) { tdma.issue_range(ly2, gy2, idx * PW / n, (idx + 1) * PW / n); };
+            const T* gy2 = Y2 + (size_t)GRAN * i * rsA;
+            auto hook = [&](int idx, int n) { tdma.issue_range(ly2, gy2, idx * PW / n, (idx + 1) * PW / n, ra); };
             gemm2(reinterpret_cast<const T*>(y2s + ((i - 1) & 1) * Cfg::TILE_BYTES), pf, hook);
         };
         int i = 1;
@@ -662,23 +674,23 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             if constexpr (MODE == R8_FWD) {
                 if (a.O) __syncthreads();   // with an output gate, the producer of the same rows takes the gated copy from here
             }
-            char* const gout = reinterpret_cast<char*>(a.out) + ((hoff + r0) * D + (size_t)dh * (D / 2)) * sizeof(T);
+            char* const gout = reinterpret_cast<char*>(a.out) + (offO + (size_t)r0 * rsO + (size_t)dh * (D / 2)) * sizeof(T);
 #pragma unroll
             for (int i = 0; i < 64 * CPR / 64; i++) {
                 const int c = lane + 64 * i, rr = c / CPR, cc = c % CPR;
                 if (r0 + rr < S)
-                    *reinterpret_cast<uint4*>(gout + (size_t)rr * D * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + rr * RB + 16 * cc);
+                    *reinterpret_cast<uint4*>(gout + (size_t)rr * rsO * sizeof(T) + 16 * cc) = *reinterpret_cast<const uint4*>(stage + rr * RB + 16 * cc);
             }
         }
     }
 #endif
 }
 
-template <typename T, int D, int MODE>
+template <typename T, int D, int MODE, bool DENSE>
 static int launch_row8_t(const RowArgs& a, hipStream_t st) {
     using Cfg = Row8Cfg<T, D>;
-    auto kern = row8_kernel<T, D, MODE>;
-    if (hipError_t e = lds_limit_once<row8_kernel<T, D, MODE>>(160 * 1024); e != hipSuccess) return (int)e;
+    auto kern = row8_kernel<T, D, MODE, DENSE>;
+    if (hipError_t e = lds_limit_once<row8_kernel<T, D, MODE, DENSE>>(160 * 1024); e != hipSuccess) return (int)e;
     const size_t lds = Cfg::FIXED_BYTES + (size_t)a.NG * sizeof(double);
     if (lds > 160 * 1024) return MLSTM_ESHAPE;  // caller falls back to the four-wave kernel
     const int nQT = (a.S + R8_BQ - 1) / R8_BQ;
@@ -686,21 +698,22 @@ static int launch_row8_t(const RowArgs& a, hipStream_t st) {
     return (int)hipGetLastError();
 }
 
-template <typename T>
+template <typename T, bool DENSE>
 static int launch_row8_m(int mode, int D, const RowArgs& a, hipStream_t st) {
     if (mode == R8_FWD) {
-        if (D == 128) return launch_row8_t<T, 128, R8_FWD>(a, st);
-        if (D == 256) return launch_row8_t<T, 256, R8_FWD>(a, st);
+        if (D == 128) return launch_row8_t<T, 128, R8_FWD, DENSE>(a, st);
+        if (D == 256) return launch_row8_t<T, 256, R8_FWD, DENSE>(a, st);
     } else {
-        if (D == 128) return launch_row8_t<T, 128, R8_DQ>(a, st);
-        if (D == 256) return launch_row8_t<T, 256, R8_DQ>(a, st);
+        if (D == 128) return launch_row8_t<T, 128, R8_DQ, DENSE>(a, st);
+        if (D == 256) return launch_row8_t<T, 256, R8_DQ, DENSE>(a, st);
     }
     return MLSTM_ESHAPE;
 }
 
 int launch_row8_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st) {
-    if (dtype == MLSTM_F16) return launch_row8_m<_Float16>(mode, D, a, st);
-    if (dtype == MLSTM_BF16) return launch_row8_m<__bf16>(mode, D, a, st);
+    const bool dense = is_dense(a.la, a.S, D) && is_dense(a.lb, a.S, D) && (mode == R8_FWD || is_dense(a.lh, a.S, D));
+    if (dtype == MLSTM_F16) return dense ? launch_row8_m<_Float16, true>(mode, D, a, st) : launch_row8_m<_Float16, false>(mode, D, a, st);
+    if (dtype == MLSTM_BF16) return dense ? launch_row8_m<__bf16, true>(mode, D, a, st) : launch_row8_m<__bf16, false>(mode, D, a, st);
     return MLSTM_ESHAPE;
 }
 

@@ -5,6 +5,12 @@ Mirror of the reference module mlstm_matmul.py: ``Triton_mLSTM.apply(q, k, v, f,
 ``SB`` and ``num_warps`` are accepted and ignored: tiling is fixed by the kernels and results do not depend on it.
 Outputs follow the inputs: h and dq, dk, dv have q's dtype (fp32 for fp32 inputs, as in the reference),
 df and di have f's dtype, the saved m and b are fp32.
+
+Beyond the reference: q, k, v need not be contiguous [B,NH,S,D].  Any [B,NH,S,D] view whose head dimension is
+contiguous is taken as it is (``x.view(B, S, NH, D).transpose(1, 2)`` of a projection's output, or the three slices of
+a fused q/k/v projection), h comes back in the same dimension order and every gradient in the layout of its tensor;
+``gate_form`` lets f arrive as its log-sigmoid or as the cumulative sum of that (the step the reference's
+cutlass-src-hopper/mlstm_forward.cu:201 suggests fusing into the projection).  The gated variants take dense tensors.
 """
 import torch
 
@@ -12,14 +18,17 @@ from . import _ffi
 
 
 def _check_inputs(q, k, v, f, i, precise=False):
+    """Shapes, dtypes and layouts.  q, k, v: [B,NH,S,D] with a contiguous head dimension and one common layout
+    otherwise (a [B,S,NH,D] projection viewed through transpose(1, 2), slices of a fused q/k/v projection, or plain
+    contiguous tensors: the kernels address rows through the strides, nothing is copied); f, i: [B,NH,S], any strides."""
     if q.dim() != 4:
         raise ValueError(f"q must be [B, NH, S, D], got {tuple(q.shape)}")
     B, NH, S, D = q.shape
-    _ffi.require(q, "q")
-    _ffi.require(k, "k", q.shape)
-    _ffi.require(v, "v", q.shape)
-    _ffi.require(f, "f", (B, NH, S))
-    _ffi.require(i, "i", (B, NH, S))
+    _ffi.require_rows(q, "q")
+    _ffi.require_rows(k, "k", q.shape, like=q)
+    _ffi.require_rows(v, "v", q.shape, like=q)
+    _ffi.require_rows(f, "f", (B, NH, S))
+    _ffi.require_rows(i, "i", (B, NH, S), like=f)
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise TypeError("q, k, v must share one dtype")
     if i.dtype != f.dtype:
@@ -27,69 +36,96 @@ def _check_inputs(q, k, v, f, i, precise=False):
     return B, NH, S, D, _ffi.dtype_code(q.dtype, precise), _ffi.dtype_code(f.dtype)
 
 
-def mlstm_forward_hip(q, k, v, f, i, precise=False):
-    """Returns (h, m, b): h [B,NH,S,D] in q's dtype, m and b [B,NH,S] fp32 (reference mlstm_matmul.py:373-378)."""
+def _dh_like(dh, h):
+    """dh in h's layout (the kernels read h and dh through one set of strides)."""
+    if tuple(dh.stride()) == tuple(h.stride()):
+        return dh
+    out = _ffi.strided_like(h)[0]
+    out.copy_(dh)
+    return out
+
+
+def mlstm_forward_hip(q, k, v, f, i, precise=False, gate_form="raw"):
+    """Returns (h, m, b): h [B,NH,S,D] in q's dtype and dimension order in memory, m and b [B,NH,S] fp32 (reference
+    mlstm_matmul.py:373-378).  gate_form: what f holds ("raw" pre-activations as in the reference, "logsigmoid", or
+    "cumsum" of the log-sigmoid over the positions; fp32 gates only for the last)."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
-    h = torch.empty_like(q)
+    h = _ffi.dense_in_order_of(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     b = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
+    lay = _ffi.layout(q, h, f, gate_form)
     ws, n = _ffi.workspace(_ffi.OP_FORWARD, B, NH, S, D, dt, q.device)
-    rc = _ffi.lib().mlstm_forward_ex(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h), _ffi.ptr(m),
-                                     _ffi.ptr(b), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n, _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_forward_ex")
+    rc = _ffi.lib().mlstm_forward_lx(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h), _ffi.ptr(m),
+                                     _ffi.ptr(b), B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n, _ffi.stream_ptr())
+    _ffi.check_rc(rc, "mlstm_forward_lx")
     return h, m, b
 
 
-def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False):
-    """Returns (dq, dk, dv, df, di) (reference mlstm_matmul.py:384-405).  h, m, b: the forward's outputs, or None
-    to have them recomputed."""
+def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False, gate_form="raw"):
+    """Returns (dq, dk, dv, df, di) (reference mlstm_matmul.py:384-405), each in the layout of the tensor it is the
+    gradient of; df is the gradient of whatever f held (gate_form).  h, m, b: the forward's outputs, or None to have
+    them recomputed."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
-    _ffi.require(dh, "dh", q.shape)
+    if not dh.is_cuda or tuple(dh.shape) != tuple(q.shape):
+        raise ValueError(f"dh must be a GPU tensor of q's shape, got {tuple(dh.shape)} on {dh.device}")
     if dh.dtype != q.dtype:
         raise TypeError("dh must have q's dtype")
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    df, di = torch.empty_like(f), torch.empty_like(i)
-    ws, n = _ffi.workspace(_ffi.OP_BACKWARD, B, NH, S, D, dt, q.device)
     if h is None or m is None or b is None:
         h = m = b = None
-    rc = _ffi.lib().mlstm_backward_ex(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h),
+        if dh.stride(-1) != 1 and D > 1:   # (an expanded or transposed gradient: one copy, into q's dimension order)
+            dh = _dh_like(dh, _ffi.dense_in_order_of(q))
+        out_like = dh   # (the recomputed h is the library's own; dh is read through its own strides)
+    else:
+        _ffi.require_rows(h, "h", q.shape)
+        dh = _dh_like(dh, h)
+        out_like = h
+    dq, dk, dv = _ffi.strided_like(q, 3)
+    df, di = _ffi.strided_like(f, 2)
+    lay = _ffi.layout(q, out_like, f, gate_form)
+    ws, n = _ffi.workspace(_ffi.OP_BACKWARD, B, NH, S, D, dt, q.device)
+    rc = _ffi.lib().mlstm_backward_lx(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h),
                                       _ffi.ptr(m), _ffi.ptr(b), _ffi.ptr(dq), _ffi.ptr(dk), _ffi.ptr(dv), _ffi.ptr(df),
-                                      _ffi.ptr(di), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n, _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_backward_ex")
+                                      _ffi.ptr(di), B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n, _ffi.stream_ptr())
+    _ffi.check_rc(rc, "mlstm_backward_lx")
     return dq, dk, dv, df, di
 
 
-def mlstm_forward_save_hip(q, k, v, f, i, precise=False):
+def mlstm_forward_save_hip(q, k, v, f, i, precise=False, gate_form="raw"):
     """Forward of a training step.  Returns (h, m, b, saved): as mlstm_forward_hip, plus what the backward can reuse (the
     states at the chunk ends of a long 16-bit sequence; None for shapes that do not run in chunks)."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
-    h = torch.empty_like(q)
+    h = _ffi.dense_in_order_of(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     b = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     nsaved = int(_ffi.lib().mlstm_saved_state_bytes(B, NH, S, D, dt))
     saved = torch.empty(nsaved, dtype=torch.uint8, device=q.device) if nsaved else None
+    lay = _ffi.layout(q, h, f, gate_form)
     ws, n = _ffi.workspace(_ffi.OP_FORWARD, B, NH, S, D, dt, q.device)
-    rc = _ffi.lib().mlstm_forward_save_ex(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h), _ffi.ptr(m),
-                                          _ffi.ptr(b), _ffi.ptr(saved), nsaved, B, NH, S, D, dt, gdt, _ffi.ptr(ws), n,
+    rc = _ffi.lib().mlstm_forward_save_lx(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h), _ffi.ptr(m),
+                                          _ffi.ptr(b), _ffi.ptr(saved), nsaved, B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n,
                                           _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_forward_save_ex")
+    _ffi.check_rc(rc, "mlstm_forward_save_lx")
     return h, m, b, saved
 
 
-def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=False):
+def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=False, gate_form="raw"):
     """Backward of a training step with the forward's outputs and its saved states (mlstm_forward_save_hip)."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
-    _ffi.require(dh, "dh", q.shape)
+    if not dh.is_cuda or tuple(dh.shape) != tuple(q.shape):
+        raise ValueError(f"dh must be a GPU tensor of q's shape, got {tuple(dh.shape)} on {dh.device}")
+    _ffi.require_rows(h, "h", q.shape)
     if dh.dtype != q.dtype:
         raise TypeError("dh must have q's dtype")
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    df, di = torch.empty_like(f), torch.empty_like(i)
+    dh = _dh_like(dh, h)
+    dq, dk, dv = _ffi.strided_like(q, 3)
+    df, di = _ffi.strided_like(f, 2)
+    lay = _ffi.layout(q, h, f, gate_form)
     ws, n = _ffi.workspace(_ffi.OP_BACKWARD, B, NH, S, D, dt, q.device)
     nsaved = 0 if saved is None else saved.numel()
-    rc = _ffi.lib().mlstm_backward_saved_ex(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h),
+    rc = _ffi.lib().mlstm_backward_saved_lx(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(h),
                                             _ffi.ptr(m), _ffi.ptr(b), _ffi.ptr(saved), nsaved, _ffi.ptr(dq), _ffi.ptr(dk), _ffi.ptr(dv),
-                                            _ffi.ptr(df), _ffi.ptr(di), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n, _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_backward_saved_ex")
+                                            _ffi.ptr(df), _ffi.ptr(di), B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n, _ffi.stream_ptr())
+    _ffi.check_rc(rc, "mlstm_backward_saved_lx")
     return dq, dk, dv, df, di
 
 
@@ -102,18 +138,21 @@ class Triton_mLSTM(torch.autograd.Function):
     """Drop-in for the reference's autograd function of the same name (mlstm_matmul.py:368-405)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, f, i, SB=16, num_warps=8):
-        h, m, b, saved = mlstm_forward_save_hip(q, k, v, f, i)
+    def forward(ctx, q, k, v, f, i, SB=16, num_warps=8, gate_form="raw"):
+        h, m, b, saved = mlstm_forward_save_hip(q, k, v, f, i, gate_form=gate_form)
         ctx.save_for_backward(q, k, v, f, i, m, b, h, saved)
         ctx.sb = SB
+        ctx.gate_form = gate_form
         return h
 
     @staticmethod
     def backward(ctx, dh):
-        assert dh.is_contiguous()
+        # (the reference asserts dh.is_contiguous(), mlstm_matmul.py:385; here every layout with a contiguous head
+        # dimension is taken as it is, e.g. the gradient of a [B,S,NH,D] view)
+        assert dh.stride(-1) == 1 or dh.shape[-1] == 1
         q, k, v, f, i, m, b, h, saved = ctx.saved_tensors
-        dq, dk, dv, df, di = mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved)
-        return dq, dk, dv, df, di, None, None
+        dq, dk, dv, df, di = mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, gate_form=ctx.gate_form)
+        return dq, dk, dv, df, di, None, None, None
 
 
 HIP_mLSTM = Triton_mLSTM
@@ -126,18 +165,21 @@ class Triton_mLSTM_precise(torch.autograd.Function):
     many MFMAs again.  Same call signature."""
 
     @staticmethod
-    def forward(ctx, q, k, v, f, i, SB=16, num_warps=8):
-        h, m, b, saved = mlstm_forward_save_hip(q, k, v, f, i, precise=True)
+    def forward(ctx, q, k, v, f, i, SB=16, num_warps=8, gate_form="raw"):
+        h, m, b, saved = mlstm_forward_save_hip(q, k, v, f, i, precise=True, gate_form=gate_form)
         ctx.save_for_backward(q, k, v, f, i, m, b, h, saved)
         ctx.sb = SB
+        ctx.gate_form = gate_form
         return h
 
     @staticmethod
     def backward(ctx, dh):
-        assert dh.is_contiguous()
+        # (the reference asserts dh.is_contiguous(), mlstm_matmul.py:385; here every layout with a contiguous head
+        # dimension is taken as it is, e.g. the gradient of a [B,S,NH,D] view)
+        assert dh.stride(-1) == 1 or dh.shape[-1] == 1
         q, k, v, f, i, m, b, h, saved = ctx.saved_tensors
-        dq, dk, dv, df, di = mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=True)
-        return dq, dk, dv, df, di, None, None
+        dq, dk, dv, df, di = mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=True, gate_form=ctx.gate_form)
+        return dq, dk, dv, df, di, None, None, None
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -149,6 +191,8 @@ class Triton_mLSTM_precise(torch.autograd.Function):
 def mlstm_forward_gated_hip(q, k, v, f, i, o):
     """Returns (h_gated, h, m, b); h is the ungated output, which the backward needs."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    for name, t in (("q", q), ("k", k), ("v", v), ("f", f), ("i", i)):
+        _ffi.require(t, name)   # the gated entry points take dense tensors
     _ffi.require(o, "o", q.shape)
     if o.dtype != q.dtype:
         raise TypeError("o must have q's dtype")
@@ -166,6 +210,8 @@ def mlstm_forward_gated_hip(q, k, v, f, i, o):
 def mlstm_backward_gated_hip(dhg, q, k, v, f, i, o, h=None, m=None, b=None):
     """Returns (dq, dk, dv, df, di, do) for the gradient dhg of the gated output."""
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
+    for name, t in (("q", q), ("k", k), ("v", v), ("f", f), ("i", i)):
+        _ffi.require(t, name)   # the gated entry points take dense tensors
     _ffi.require(o, "o", q.shape)
     _ffi.require(dhg, "dh", q.shape)
     if dhg.dtype != q.dtype or o.dtype != q.dtype:
@@ -175,6 +221,8 @@ def mlstm_backward_gated_hip(dhg, q, k, v, f, i, o, h=None, m=None, b=None):
     ws, n = _ffi.workspace(_ffi.OP_BACKWARD_GATED, B, NH, S, D, dt, q.device)
     if h is None or m is None or b is None:
         h = m = b = None
+    else:
+        _ffi.require(h, "h", q.shape)
     rc = _ffi.lib().mlstm_backward_gated_ex(_ffi.ptr(dhg), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o),
                                             _ffi.ptr(h), _ffi.ptr(m), _ffi.ptr(b), _ffi.ptr(dq), _ffi.ptr(dk), _ffi.ptr(dv),
                                             _ffi.ptr(df), _ffi.ptr(di), _ffi.ptr(do), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n,
