@@ -98,8 +98,14 @@ int mlstm_backward(const void* dH, const void* Q, const void* K, const void* V, 
  * General forward: what Triton_mLSTM.forward / mlstm_matmul launch,
  *   mlstm_matmul_kernel[grid](q,k,v,f,i,m,b,h,NH,S,D,SB)        (mlstm_matmul.py:38-101, :121-129, :371-381).
  * dtype is the element type of q, k, v and h; gate_dtype that of f and i; m and b are always fp32.
- * D in {64,128,256} (fp32: {64,128}); any S >= 1.  workspace may be NULL (the library then allocates and
- * frees stream-ordered); otherwise it must hold mlstm_workspace_bytes(MLSTM_OP_FORWARD, ...) bytes.
+ * D in {64,128,256} for fp16 / bf16, {64,...,1024} (powers of two) for fp32; any S >= 1.  fp32 at D >= 256 runs on
+ * the scan form's kernels (same function, see mlstm_scan_forward_ex): the tile kernels hold a row block's D columns
+ * in accumulator registers and two D-wide tiles per stage in LDS, which ends at D = 128 in fp32 and at D = 256 in
+ * 16 bits; a D = 512 16-bit variant would need the head dimension tiled as well (a second kernel family), and is not
+ * built.  At those fp32 sizes the tensors must be dense, the gates fp32 pre-activations, and the backward recomputes
+ * the forward (h, m, b are ignored); the gated entry points and layouts of the caller's return MLSTM_ESHAPE there.
+ * workspace may be NULL (the library then allocates and frees stream-ordered); otherwise it must hold
+ * mlstm_workspace_bytes(MLSTM_OP_FORWARD, ...) bytes.
  */
 int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m,
                      float* b, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace,

@@ -65,7 +65,8 @@ def test_workspace_sizes_and_argument_errors_need_no_gpu():
     one = ctypes.c_void_p(16)  # never dereferenced: the shape check comes first
     assert L.mlstm_forward_ex(null, null, null, null, null, null, null, null, 1, 1, 64, 64, ffi.F32, ffi.F32, null, 0, null) == -1
     assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 48, ffi.F32, ffi.F32, null, 0, null) == -2
-    assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 256, ffi.F32, ffi.F32, null, 0, null) == -2
+    assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 512, ffi.BF16, ffi.F32, null, 0, null) == -2
+    assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 2048, ffi.F32, ffi.F32, null, 0, null) == -2
     assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 64, 9, ffi.F32, null, 0, null) == -1
     assert L.mlstm_forward_ex(one, one, one, one, one, one, null, null, 1, 1, 64, 64, ffi.F32, ffi.F32, one, 8, null) == -3
     assert L.mlstm_backward_ex(*([one] * 6), null, null, null, *([one] * 5), 1, 1, 64, 96, ffi.F16, ffi.F16, null, 0, null) == -2

@@ -102,3 +102,31 @@ def test_scan_backward_rejects_what_it_cannot_serve():
     x96 = [t.cuda() for t in O.make_inputs(1, 1, 64, 96, torch.float32, seed=1, with_o=True)]
     with pytest.raises(ValueError):   # a head dimension the scan kernels are not built for
         mlstm_scan_backward_hip(x96[5], x96[0], x96[1], x96[2], x96[3], x96[4], x96[6])
+
+
+@pytest.mark.parametrize("S,D", [(300, 256), (200, 512), (130, 1024)])
+def test_matmul_form_fp32_at_large_head_dimensions(S, D):
+    # fp32 at D >= 256: the matmul form's entry points (forward with m and b, backward, the autograd function) run on
+    # the scan kernels; checked against the dense oracle of the matmul form
+    from mlstm_matmul import Triton_mLSTM, mlstm_backward_hip, mlstm_forward_hip
+    q, k, v, f, i, dh = O.make_inputs(1, 2, S, D, torch.float32, seed=S + D)
+    dev = [x.cuda() for x in (q, k, v, f, i)]
+    h, m, b = mlstm_forward_hip(*dev)
+    hr, mr, br = O.mlstm_forward_dense(q, k, v, f, i)
+    assert_close(h, hr, torch.float32, "h")
+    assert_close(m, mr, torch.float32, "m")
+    assert_close(b, br, torch.float32, "b")
+    ref = O.mlstm_backward_dense(dh, q, k, v, f, i, zero_first_df=True)
+    for name, g, r in zip(NAMES, mlstm_backward_hip(dh.cuda(), *dev), ref):
+        assert_close(g, r, torch.float32, name)
+    leaves = [x.clone().requires_grad_(True) for x in dev]
+    Triton_mLSTM.apply(*leaves).backward(dh.cuda())
+    for name, x, r in zip(NAMES, leaves, ref):
+        assert_close(x.grad, r, torch.float32, "autograd " + name)
+
+
+def test_matmul_form_fp32_large_head_dimension_limits():
+    from mlstm_matmul import mlstm_forward_hip
+    q, k, v, f, i, _ = (x.cuda() for x in O.make_inputs(1, 2, 128, 256, torch.float32, seed=2))
+    with pytest.raises(ValueError):      # a layout of the caller's: dense tensors only at these sizes
+        mlstm_forward_hip(*(x.transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v)), f, i)

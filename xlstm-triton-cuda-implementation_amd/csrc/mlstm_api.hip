@@ -89,9 +89,18 @@ struct Sizes {
     // what the backward reuses of the forward: in chunks the value-major states, the vector states and the gate
     // pre-pass; in split mode h - (h rounded to the element type)
     size_t saved() const { return precise ? h_lo() : (n_states(chunk_len()) ? states_t() + saved_vec() + gates() : 0); }
-    size_t fwd() const { return gates() + stats() + chunk_states(dtype_code); }
+    // fp32 at head dimensions of 256 and more: the matmul form's entry points run on the scan form's kernels (the same
+    // function; the tile kernels' accumulators and LDS stages end at D = 128 in fp32)
+    bool scan_engine() const { return dtype_code == MLSTM_F32 && D >= 256; }
+    // scan form: gates, m, row sums, in-chunk pairs, vector states, partial numerators of the other key ranges
+    size_t scan_fwd() const {
+        return gates() + stats() + up256(BH * NG * 64 * 64 * 4) + up256(BH * NG * D * 4) +
+               (size_t)(scan_key_splits((int)BH, (int)D) - 1) * up256(BH * S * D * 4);
+    }
+    size_t fwd() const { return scan_engine() ? scan_fwd() : gates() + stats() + chunk_states(dtype_code); }
     size_t fwd_fixed() const { return gates() + stats(); }   // offset of the chunk states inside fwd()
     size_t bwd() const {
+        if (scan_engine()) return scan_backward_workspace_bytes((int)BH, (int)S, (int)D);
         return fwd() + up256(BH * S * D * el)                                      // recomputed h
                + 2 * up256(BH * NG * 64 * 4) + states_t()                          // inv_n, db; transposed chunk states
                + states_t() + saved_vec() + up256(BH * S * 4)                      // reverse states (value-major, vector); far row sums
@@ -123,7 +132,7 @@ Sizes sizes_of(int B, int NH, int S, int D, int dtype_arg) {
     z.lg = dense_layout(NH, S, 1);
     return z;
 }
-bool good_shape(int D, int dtype) { return D == 64 || D == 128 || (D == 256 && dtype != MLSTM_F32); }
+bool good_shape(int D, int dtype) { return D == 64 || D == 128 || D == 256 || (dtype == MLSTM_F32 && (D == 512 || D == 1024)); }
 
 // The caller's layout into z (null: everything dense).  Rows of q, k, v, h must start on 16-byte boundaries, and the
 // tile copies address a tile's 64 rows with 32-bit byte offsets.
@@ -241,11 +250,49 @@ int chunk_states_impl(const void* k, const void* v, const FwdWs& w, bool key_maj
     return launch_chunk_states(dtype, D, ca, st);
 }
 
+// The scan form's pipeline on a workspace of Sizes::scan_fwd() bytes: gate pre-pass, in-chunk pairs and vector carry,
+// matrix state walk, finish.  finish_mode as in ScanArgs; m_out / b_out (may be null) receive the stabiliser and the
+// normaliser sums.
+int scan_forward_impl(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h, float* m_out,
+                      float* b_out, const Sizes& z, int gate_dtype, int finish_mode, char* ws, hipStream_t st) {
+    Carver c{ws, 0};
+    double* G2 = c.take<double>(z.BH * z.NG);
+    float* alpha2 = c.take<float>(z.BH * z.NG * 64);
+    float* beta2 = c.take<float>(z.BH * z.NG * 64);
+    float* ek2 = c.take<float>(z.BH * z.NG * 64);
+    float* amax2 = c.take<float>(z.BH * z.NG * 2 + 64);   // (+64: the row kernels copy 64 floats from each tile's pair on)
+    float* m = c.take<float>(z.BH * z.S);
+    float* bw = c.take<float>(z.BH * z.S);
+    float* P = c.take<float>(z.BH * z.NG * 64 * 64);
+    float* Nst = c.take<float>(z.BH * z.NG * z.D);
+    const int KS = scan_key_splits((int)z.BH, (int)z.D);
+    float* hpart = nullptr;
+    for (int p = 1; p < KS; p++) { float* x = c.take<float>(z.BH * z.S * z.D); if (p == 1) hpart = x; }
+    if (m_out) m = m_out;
+    (void)bw;
+    {
+        Timed t(MLSTM_K_GATES, st);
+        hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st, z.lg, z.gate_form);
+        if (e != hipSuccess) return (int)e;
+    }
+    ScanArgs a{};
+    a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v; a.o = (const float*)o; a.h = (float*)h;
+    a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.P = P; a.Nst = Nst; a.hpart = hpart;
+    a.BH = (int)z.BH; a.S = (int)z.S; a.D = (int)z.D; a.NC = (int)z.NG;
+    a.finish_mode = finish_mode; a.Bout = b_out;
+    return launch_scan(a, KS, st, scan_mark);
+}
+
 int forward_impl(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m, float* b,
                  const Sizes& z, int D, int dtype, int gate_dtype, char* ws, hipStream_t st, float** alpha_out = nullptr,
                  float** beta_out = nullptr, double** g_out = nullptr, float** m_out = nullptr, float** b_out = nullptr,
                  float** ek_out = nullptr, float** amax_out = nullptr, const void* o = nullptr, void* h_gated = nullptr,
                  void* CstT = nullptr, float* Nst_ext = nullptr, char* gates_ext = nullptr, void* h_lo = nullptr) {
+    if (z.scan_engine()) {
+        // dense tensors only, no fused gate copy (mlstm_scan_forward_ex is the gated form of these kernels)
+        if (o || h_gated || !is_dense(z.la, (long long)z.S, (long long)z.D) || !is_dense(z.lb, (long long)z.S, (long long)z.D)) return MLSTM_ESHAPE;
+        return scan_forward_impl(q, k, v, f, i, nullptr, h, m, b, z, gate_dtype, 1, ws, st);
+    }
     FwdWs w(ws, z, dtype, D);
     if (gates_ext) w.gates_at(gates_ext, z);
     double* G2 = w.G2; float *alpha2 = w.alpha2, *beta2 = w.beta2, *ek2 = w.ek2, *amax2 = w.amax2;
@@ -363,9 +410,7 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype) {
         case MLSTM_OP_BACKWARD: return z.bwd();
         case MLSTM_OP_FORWARD_GATED: return z.fwd();
         case MLSTM_OP_BACKWARD_GATED: return z.bwd_gated();
-        case MLSTM_OP_SCAN_FORWARD:  // gates, m, row sums, in-chunk pairs, vector states, partial numerators
-            return z.fwd() + up256(z.BH * z.NG * 64 * 64 * 4) + up256(z.BH * z.NG * z.D * 4) +
-                   (size_t)(scan_key_splits((int)z.BH, D) - 1) * up256(z.BH * z.S * z.D * 4);
+        case MLSTM_OP_SCAN_FORWARD: return z.scan_fwd();
         case MLSTM_OP_SCAN_BACKWARD:
             return (D % 64 == 0 && D >= 64) ? scan_backward_workspace_bytes((int)z.BH, S, D) : 0;
     }
@@ -471,6 +516,17 @@ namespace {
 int backward_impl(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h, const float* m,
                   const float* b, void* dq, void* dk, void* dv, void* df, void* di, const Sizes& z, int D, int dtype, int gate_dtype,
                   char* ws, hipStream_t st, const char* saved = nullptr) {
+    if (z.scan_engine()) {   // (recomputes the forward it needs; h, m, b are not read)
+        if (!is_dense(z.la, (long long)z.S, (long long)z.D) || !is_dense(z.lb, (long long)z.S, (long long)z.D) ||
+            !is_dense(z.lg, (long long)z.S, 1) || z.gate_form != MLSTM_GATE_RAW || gate_dtype != MLSTM_F32)
+            return MLSTM_ESHAPE;
+        ScanBwdArgs a{};
+        a.dhg = (const float*)dh; a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v;
+        a.f = (const float*)f; a.i = (const float*)i; a.o = nullptr;
+        a.dq = (float*)dq; a.dk = (float*)dk; a.dv = (float*)dv; a.df = (float*)df; a.di = (float*)di; a.d_o = nullptr;
+        a.BH = (int)z.BH; a.S = (int)z.S; a.D = D;
+        return launch_scan_backward(a, ws, st, scan_mark);
+    }
     Carver c{ws, z.fwd()};
     char* hbuf = c.take<char>(z.BH * z.S * z.D * z.el);
     float* inv_n = c.take<float>(z.BH * z.NG * 64);
@@ -666,33 +722,10 @@ int mlstm_scan_forward_ex(const void* q, const void* k, const void* v, const voi
     if (dtype != MLSTM_F32) return MLSTM_ESHAPE;  // the scan form is fp32, like the reference's
     if (!(D == 64 || D == 128 || D == 256 || D == 512 || D == 1024) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    Sizes z{(size_t)B * NH, (size_t)S, (size_t)D, (size_t)(S + GATE_GRANULE - 1) / GATE_GRANULE, 4};
-    const size_t need = mlstm_workspace_bytes(MLSTM_OP_SCAN_FORWARD, B, NH, S, D, dtype);
+    const Sizes z = sizes_of(B, NH, S, D, MLSTM_F32);
     Scratch sc;
-    if (int rc = sc.get(workspace, workspace_bytes, need, st)) return rc;
-    Carver c{(char*)sc.p, 0};
-    double* G2 = c.take<double>(z.BH * z.NG);
-    float* alpha2 = c.take<float>(z.BH * z.NG * 64);
-    float* beta2 = c.take<float>(z.BH * z.NG * 64);
-    float* ek2 = c.take<float>(z.BH * z.NG * 64);
-    float* amax2 = c.take<float>(z.BH * z.NG * 2 + 64);   // (+64: the row kernels copy 64 floats from each tile's pair on)
-    float* m = c.take<float>(z.BH * z.S);
-    c.take<float>(z.BH * z.S);  // (the matmul form keeps its normaliser sums here)
-    float* P = c.take<float>(z.BH * z.NG * 64 * 64);
-    float* Nst = c.take<float>(z.BH * z.NG * z.D);
-    const int KS = scan_key_splits((int)z.BH, D);
-    float* hpart = nullptr;
-    for (int p = 1; p < KS; p++) { float* x = c.take<float>(z.BH * z.S * z.D); if (p == 1) hpart = x; }
-    {
-        Timed t(MLSTM_K_GATES, st);
-        hipError_t e = launch_gates(MLSTM_F32, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st);
-        if (e != hipSuccess) return (int)e;
-    }
-    ScanArgs a{};
-    a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v; a.o = (const float*)o; a.h = (float*)h;
-    a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.P = P; a.Nst = Nst; a.hpart = hpart;
-    a.BH = (int)z.BH; a.S = (int)z.S; a.D = D; a.NC = (int)z.NG;
-    return launch_scan(a, KS, st, scan_mark);
+    if (int rc = sc.get(workspace, workspace_bytes, z.scan_fwd(), st)) return rc;
+    return scan_forward_impl(q, k, v, f, i, o, h, nullptr, nullptr, z, MLSTM_F32, 0, (char*)sc.p, st);
 }
 
 int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,

@@ -200,7 +200,8 @@ int launch_scan(const ScanArgs& a, int KS, hipStream_t st, void (*mark)(int, hip
 void launch_scan_ncarry(const ScanArgs& a, hipStream_t st);
 
 // Backward of the scan form (mlstm_scan_bwd.hip): every pointer fp32, [B,NH,S,D] or [B,NH,S]; ws holds
-// scan_backward_workspace_bytes(BH, S, D) bytes
+// scan_backward_workspace_bytes(BH, S, D) bytes.  o == null: no output gate (dhg is the gradient of the ungated
+// output, d_o is not written)
 struct ScanBwdArgs {
     const float* dhg; const float* q; const float* k; const float* v; const float* f; const float* i; const float* o;
     float* dq; float* dk; float* dv; float* df; float* di; float* d_o;

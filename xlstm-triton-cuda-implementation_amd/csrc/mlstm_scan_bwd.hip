@@ -275,7 +275,7 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
     const Plan p = plan_of(ws, BH, S, D);
     const size_t rows = (size_t)BH * S, N = rows * D;
     const int KS = scan_key_splits(BH, D), rb = row_blocks(rows);
-    float *h = p.T[0], *dh = p.T[1], *u = p.T[2], *yloc = p.T[3], *qr = p.T[4], *kr = p.T[5], *vr = p.T[6], *ur = p.T[7];
+    float *h = p.T[0], *u = p.T[2], *yloc = p.T[3], *qr = p.T[4], *kr = p.T[5], *vr = p.T[6], *ur = p.T[7];
     float *RV = p.T[0], *RK = p.T[1];  // (h and dh are done with by then)
 
     mark(MLSTM_K_GATES, st, true);
@@ -295,10 +295,16 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
         s.q = a.q; s.k = a.k; s.v = a.v; s.h = h; s.finish_mode = 1; s.Bout = p.b;
         if (int rc = launch_scan(s, KS, st, mark)) return rc;
     }
-    mark(MLSTM_K_GATE_BWD, st, true);
-    const int gb = launch_gate_backward(MLSTM_F32, a.dhg, a.o, h, dh, a.d_o, N, st);
-    mark(MLSTM_K_GATE_BWD, st, false);
-    if (gb) return gb;
+    // the gradient of the ungated output: through the gate's backward, or, without a gate (o == null: the matmul
+    // form's backward at head dimensions only these kernels serve), the caller's own
+    const float* dh = a.dhg;
+    if (a.o) {
+        mark(MLSTM_K_GATE_BWD, st, true);
+        const int gb = launch_gate_backward(MLSTM_F32, a.dhg, a.o, h, p.T[1], a.d_o, N, st);
+        mark(MLSTM_K_GATE_BWD, st, false);
+        if (gb) return gb;
+        dh = p.T[1];
+    }
 
     mark(MLSTM_K_SCAN_GLUE, st, true);
     hipLaunchKernelGGL(scanbwd_rowstats_kernel, dim3(rb), dim3(256), 0, st, dh, h, p.b, p.m, u, p.db, p.db_rev, BH, S, D);
