@@ -226,11 +226,13 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
     return out, host
 
 
-def run_scan(ffi, steps, warmup, backward=False):
-    """Scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape); ``backward``: a step is the
-    forward followed by the backward (which recomputes the forward: five passes of the state kernel in all)."""
+def run_scan(ffi, steps, warmup, backward=False, shape=(1, 4, 2048, 1024), tag="cfg3"):
+    """Scan form, B1 H4 S2048 D1024 fp32 (the reference's own scan self-check shape) unless ``shape`` says otherwise;
+    ``backward``: a step is the forward followed by the backward (which recomputes the forward: five passes of the state
+    kernel in all)."""
     L = ffi.lib()
-    B, NH, S, D = 1, 4, 2048, 1024
+    B, NH, S, D = shape
+    wl = "%s_B%d_H%d_S%d_D%d_f32" % (tag, B, NH, S, D)
     dev = torch.device("cuda:0")
     host = make_inputs(B, NH, S, D, torch.float32, 0.0, 0.0, 1.0, with_o=True)
     q, k, v, f, i, dh, o = (x.to(dev) for x in host)
@@ -274,17 +276,17 @@ def run_scan(ffi, steps, warmup, backward=False):
     t_fl = flops / (st_ms * 1e-3) / 1e12 if st_ms else 0.0
     flops *= 5 if backward else 1
     return {
-        "metric": "mLSTM scan-form %s, compulsory HBM GB/s, cfg3_B1_H4_S2048_D1024_f32" % ("forward+backward" if backward else "forward"),
+        "metric": "mLSTM scan-form %s, compulsory HBM GB/s, %s" % ("forward+backward" if backward else "forward", wl),
         "value": bytes_compulsory / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "cfg3_B1_H4_S2048_D1024_f32", "B": B, "NH": NH, "S": S, "D": D},
+        "config": {"workload": wl, "B": B, "NH": NH, "S": S, "D": D},
         "tokens_per_s": B * S / (ms_step * 1e-3), "fp32_tflops": flops / (ms_step * 1e-3) / 1e12,
         "kernel_ms": {n: (t / c if c else None) for n, (t, c) in kern.items()},
         # the binding roof: 38.7 GF of fp32 matrix work against 168 MB of compulsory traffic (ridge at 20 flop/B, the
         # workload has 230); both fractions are reported
         "roofline": {"bound": "mfma", "kernel": "scan_state_kernel (fp32 MFMA)", "achieved": t_fl, "peak": 157.3, "unit": "TFLOP/s",
-                     "frac": t_fl / 157.3, "traffic": measured_traffic("cfg3_B1_H4_S2048_D1024_f32", "scan_state_kernel", 64),
+                     "frac": t_fl / 157.3, "traffic": measured_traffic(wl, "scan_state_kernel", 64),
                      "hbm_gbs": bytes_compulsory / (ms_step * 1e-3) / 1e9, "hbm_frac": bytes_compulsory / (ms_step * 1e-3) / 8e12},
     }
 
@@ -294,7 +296,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan", "cfg3_scan_backward"])
+    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan", "cfg3_scan_backward", "long_scan"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
@@ -317,6 +319,9 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    if args.workload == "long_scan":   # one long sequence: the state walk runs in segments side by side
+        print(json.dumps(run_scan(ffi, args.steps, args.warmup, shape=(1, 1, 65536, 128), tag="long")))
+        return
     if args.workload in ("cfg3_scan", "cfg3_scan_backward"):
         print(json.dumps(run_scan(ffi, args.steps, args.warmup, backward=args.workload.endswith("backward"))))
         return

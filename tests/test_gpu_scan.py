@@ -68,3 +68,22 @@ def test_scan_against_committed_golden_vector():
     g = {k_: torch.from_numpy(z[k_]) for k_ in z.files}
     h = run_scan(g["q"], g["k"], g["v"], g["f"], g["i"], g["o"])
     assert_close(h, g["h"], torch.float32, "h")
+
+
+@pytest.mark.parametrize("S,D", [(8192, 64), (3000, 64), (4096, 128), (2048, 256)])
+def test_scan_one_long_sequence_in_segments(S, D):
+    # one head: the state walk runs in segments side by side (states at the segment ends from a pass of their own);
+    # checked against the step-by-step recurrence, and against the same head inside a batch that fills the chip and
+    # therefore walks its chunks in one piece
+    q, k, v, f, i, _, o = O.make_inputs(1, 1, S, D, torch.float32, seed=S + D, with_o=True)
+    h = run_scan(q, k, v, f, i, o)
+    assert_close(h, O.mlstm_recurrent(q, k, v, f, i, o), torch.float32, "h")
+    reps = 256 // (D // 32)
+    hb = run_scan(*(x.expand(reps, *x.shape[1:]).contiguous() for x in (q, k, v, f, i, o)))
+    assert torch.equal(hb[0], hb[reps - 1])
+    assert_close(h[0], hb[0].cpu(), torch.float32, "h against the unsegmented walk")
+
+
+def test_scan_strong_forgetting_across_segments():
+    q, k, v, f, i, _, o = O.make_inputs(1, 2, 4096, 64, torch.float32, seed=77, f_mean=-3.0, with_o=True)
+    assert_close(run_scan(q, k, v, f, i, o), O.mlstm_recurrent(q, k, v, f, i, o), torch.float32, "h")

@@ -130,3 +130,10 @@ def test_matmul_form_fp32_large_head_dimension_limits():
     q, k, v, f, i, _ = (x.cuda() for x in O.make_inputs(1, 2, 128, 256, torch.float32, seed=2))
     with pytest.raises(ValueError):      # a layout of the caller's: dense tensors only at these sizes
         mlstm_forward_hip(*(x.transpose(1, 2).contiguous().transpose(1, 2) for x in (q, k, v)), f, i)
+
+
+@pytest.mark.parametrize("S,D", [(4096, 128), (2500, 64)])
+def test_scan_backward_one_long_sequence(S, D):
+    # one head: all five passes of the state kernel run in segments
+    q, k, v, f, i, dh, o = O.make_inputs(1, 1, S, D, torch.float32, seed=S + D, with_o=True)
+    check(run_backward(dh, q, k, v, f, i, o), dh, q, k, v, f, i, o)

@@ -95,7 +95,8 @@ struct Sizes {
     // scan form: gates, m, row sums, in-chunk pairs, vector states, partial numerators of the other key ranges
     size_t scan_fwd() const {
         return gates() + stats() + up256(BH * NG * 64 * 64 * 4) + up256(BH * NG * D * 4) +
-               (size_t)(scan_key_splits((int)BH, (int)D) - 1) * up256(BH * S * D * 4);
+               (size_t)(scan_key_splits((int)BH, (int)D) - 1) * up256(BH * S * D * 4) +
+               up256(scan_segment_state_bytes((int)BH, (int)S, (int)D));
     }
     size_t fwd() const { return scan_engine() ? scan_fwd() : gates() + stats() + chunk_states(dtype_code); }
     size_t fwd_fixed() const { return gates() + stats(); }   // offset of the chunk states inside fwd()
@@ -268,6 +269,7 @@ int scan_forward_impl(const void* q, const void* k, const void* v, const void* f
     const int KS = scan_key_splits((int)z.BH, (int)z.D);
     float* hpart = nullptr;
     for (int p = 1; p < KS; p++) { float* x = c.take<float>(z.BH * z.S * z.D); if (p == 1) hpart = x; }
+    float* seg_state = c.take<float>(scan_segment_state_bytes((int)z.BH, (int)z.S, (int)z.D) / 4);
     if (m_out) m = m_out;
     (void)bw;
     {
@@ -279,7 +281,7 @@ int scan_forward_impl(const void* q, const void* k, const void* v, const void* f
     a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v; a.o = (const float*)o; a.h = (float*)h;
     a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.P = P; a.Nst = Nst; a.hpart = hpart;
     a.BH = (int)z.BH; a.S = (int)z.S; a.D = (int)z.D; a.NC = (int)z.NG;
-    a.finish_mode = finish_mode; a.Bout = b_out;
+    a.finish_mode = finish_mode; a.Bout = b_out; a.seg_state = seg_state;
     return launch_scan(a, KS, st, scan_mark);
 }
 

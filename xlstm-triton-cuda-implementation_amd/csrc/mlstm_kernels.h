@@ -192,8 +192,14 @@ struct ScanArgs {
     // reuses with other operands in the places of q, k and v.  Bout (may be null): the normaliser sums b_t, modes 0 and 1.
     int finish_mode;
     float* Bout;
+    // segments of the sequence that the state kernel runs side by side (filled in by launch_scan from scan_segments);
+    // seg_state: scan_segment_state_bytes() bytes of scratch for the states at the segment ends, needed when nseg > 1
+    float* seg_state;
+    int nseg, seg_chunks;
 };
 int scan_key_splits(int BH, int D);
+void scan_segments(int BH, int S, int D, int* nseg, int* seg_chunks);
+size_t scan_segment_state_bytes(int BH, int S, int D);
 // mark(kernel id, stream, begin?) brackets groups of launches for the optional event timing
 int launch_scan(const ScanArgs& a, int KS, hipStream_t st, void (*mark)(int, hipStream_t, bool));
 // n~ at every chunk end from the chunks' own sums, in place (ScanArgs::Nst, beta2, G2, BH, NC, D are read)

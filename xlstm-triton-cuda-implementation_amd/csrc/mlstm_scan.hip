@@ -117,7 +117,13 @@ __global__ __launch_bounds__(256) void scan_ncarry_kernel(ScanArgs a) {
 template <int N> struct FVec { typedef float type __attribute__((ext_vector_type(N))); };
 template <> struct FVec<1> { struct type { float x; __device__ float operator[](int) const { return x; } }; };
 
-template <int D, int KS, int NW>
+// A sequence may also be cut into segments of seg_chunks chunks that run side by side (blockIdx.y), for the cases in
+// which heads x value tiles x key ranges alone leave most of the chip idle (one long sequence, small D):
+//   STATE_ONLY = true   every segment but the last walks its chunks from a zero state, updates only, and leaves the
+//                       state at its end (accumulator registers as they are) in seg_state;
+//   scan_segcarry_kernel turns those into the true states at the segment ends (a short serial sum over the segments);
+//   STATE_ONLY = false  the walk proper: segment s > 0 starts from the state at the end of segment s - 1.
+template <int D, int KS, int NW, bool STATE_ONLY>
 __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     constexpr int KPW = D / KS / NW, NKB = KPW / 32, NVT = D / 32;  // key columns per wave, in blocks of 32
     constexpr int SH = 32 / (NW * KS);                              // in-chunk contraction steps per wave
@@ -131,6 +137,7 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     const int vt = rest % NVT, ks = rest / NVT;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
     const int S = a.S, NC = a.NC;
+    const int seg = blockIdx.y, c_begin = seg * a.seg_chunks, c_end = c_begin + a.seg_chunks < NC ? c_begin + a.seg_chunks : NC;
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * NC * GRAN;
     const float* Q = a.q + hoff * D;
     const float* K = a.k + hoff * D;
@@ -177,22 +184,28 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     };
 
     f32x16 st[NKB];  // st[kb][r] = C~[v = v0 + c32][k = kbase + NKB*(8*(r/4) + 4h + r%4) + kb]
+    // a workgroup's state in seg_state: [segment][workgroup][wave][kb][r][lane]
+    const size_t seg_stride = (size_t)gridDim.x * NW * NKB * 16 * 64;
+    float* const seg_mine = a.seg_state + ((size_t)blockIdx.x * NW + wave) * NKB * 16 * 64 + lane;
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) st[kb][r] = 0.f;
+        for (int r = 0; r < 16; r++) st[kb][r] = (!STATE_ONLY && seg > 0) ? seg_mine[(size_t)(seg - 1) * seg_stride + (kb * 16 + r) * 64] : 0.f;
     kvec qreg[2][4][4];  // [query block][x][e]: Q[t][kbase + NKB*(8x + 4h + e) + 0..NKB-1]
     auto load_q = [&](int c, int tb, int x, int e) {  // (row clamped: the chunk may be the partial one)
         int t = GRAN * c + 32 * tb + c32;
         t = t < S ? t : S - 1;
         qreg[tb][x][e] = *reinterpret_cast<const kvec*>(Q + (size_t)t * D + kbase + 4 * NKB * h + NKB * (8 * x + e));
     };
+    if constexpr (!STATE_ONLY) {
 #pragma unroll
-    for (int i = 0; i < 32; i++) load_q(0, i & 1, i >> 3, (i >> 1) & 3);
+        for (int i = 0; i < 32; i++) load_q(c_begin, i & 1, i >> 3, (i >> 1) & 3);
+    }
     float rescale_cur;
+    float lg_done = 0.f;   // log2 Gamma of the last chunk whose update is in st
     {
-        const Gates g0 = gates_fetch(0);
-        gates_store(0, g0);
+        const Gates g0 = gates_fetch(c_begin);
+        gates_store(c_begin, g0);
         rescale_cur = g0.rescale;
     }
     __syncthreads();
@@ -229,6 +242,7 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[tb][r] = 0.f;
         Gates gn;
+        lg_done = lg;
         if constexpr (!LAST) gn = gates_fetch(c + 1);
         // the in-chunk products are split over all waves of all key ranges: SH contraction steps each
         const int s0 = (ks * NW + wave) * SH;
@@ -254,40 +268,46 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
         };
 #pragma unroll
         for (int g = 0; g < 16; g++) {  // g = 4x + e
-            if (g == 0) load_p();
-            if (g == 1) load_vin();
+            if constexpr (!STATE_ONLY) {
+                if (g == 0) load_p();
+                if (g == 1) load_vin();
+            }
             load_v(2 * g);
             load_v(2 * g + 1);
             if constexpr (!LAST) {
                 load_k(2 * g);
                 load_k(2 * g + 1);
             }
+            if constexpr (!STATE_ONLY) {
 #pragma unroll
-            for (int kb = 0; kb < NKB; kb++) {
-                acc[0] = mma_f32(qreg[0][g >> 2][g & 3][kb], st[kb][g], acc[0]);
-                acc[1] = mma_f32(qreg[1][g >> 2][g & 3][kb], st[kb][g], acc[1]);
+                for (int kb = 0; kb < NKB; kb++) {
+                    acc[0] = mma_f32(qreg[0][g >> 2][g & 3][kb], st[kb][g], acc[0]);
+                    acc[1] = mma_f32(qreg[1][g >> 2][g & 3][kb], st[kb][g], acc[1]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (!STATE_ONLY) {
 #pragma unroll
-        for (int tb = 0; tb < 2; tb++)
+            for (int tb = 0; tb < 2; tb++)
 #pragma unroll
-            for (int x = 0; x < 4; x++) {
-                const f32x4 dec = *reinterpret_cast<const f32x4*>(sdec + 32 * tb + 8 * x + 4 * h);
+                for (int x = 0; x < 4; x++) {
+                    const f32x4 dec = *reinterpret_cast<const f32x4*>(sdec + 32 * tb + 8 * x + 4 * h);
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[tb][4 * x + e] *= dec[e];
+                    for (int e = 0; e < 4; e++) acc[tb][4 * x + e] *= dec[e];
+                }
+            // ---- pairs inside the chunk: acc += P_c[:, this wave's keys] . V_c
+#pragma unroll
+            for (int s = 0; s < SH; s++) {
+                acc[0] = mma_f32(pa[0][s], vin[s], acc[0]);
+                acc[1] = mma_f32(pa[1][s], vin[s], acc[1]);
             }
-        // ---- pairs inside the chunk: acc += P_c[:, this wave's keys] . V_c
+            // ---- sum the partial numerators of the waves and store them (unnormalised)
 #pragma unroll
-        for (int s = 0; s < SH; s++) {
-            acc[0] = mma_f32(pa[0][s], vin[s], acc[0]);
-            acc[1] = mma_f32(pa[1][s], vin[s], acc[1]);
+            for (int tb = 0; tb < 2; tb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) red[c & 1][wave][16 * tb + r][lane] = acc[tb][r];
         }
-        // ---- sum the partial numerators of the waves and store them (unnormalised)
-#pragma unroll
-        for (int tb = 0; tb < 2; tb++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) red[c & 1][wave][16 * tb + r][lane] = acc[tb][r];
         if constexpr (!LAST) gates_store(c + 1, gn);
         // The only barrier of a chunk.  Between two barriers a wave is in the tail of one chunk or the head of the next:
         // the partial sums alternate between two buffers, the gate vectors (written a chunk ahead) between three.
@@ -319,8 +339,10 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const int i = 4 * x + e;
-                    load_q(c + 1, i & 1, i >> 3, (i >> 1) & 3);
-                    if (i < 32 / NW) sum_store(wave + NW * i);
+                    if constexpr (!STATE_ONLY) {
+                        load_q(c + 1, i & 1, i >> 3, (i >> 1) & 3);
+                        if (i < 32 / NW) sum_store(wave + NW * i);
+                    }
                     const float wv = vraw[i] * w4[e];
 #pragma unroll
                     for (int kb = 0; kb < NKB; kb++) st[kb] = mma_f32(kreg[i][kb], wv, st[kb]);  // rows = k, columns = v
@@ -329,8 +351,36 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
             }
         }
     };
-    for (int c = 0; c + 1 < NC; c++) chunk(c, std::false_type{});
-    chunk(NC - 1, std::true_type{});
+    if constexpr (STATE_ONLY) {
+        // (never the last segment: every chunk is complete and has a successor whose gates the walk fetches ahead)
+        for (int c = c_begin; c < c_end; c++) chunk(c, std::false_type{});
+        const float f = fast_exp2(lg_done);   // st = C~ / Gamma
+#pragma unroll
+        for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) seg_mine[(size_t)seg * seg_stride + (kb * 16 + r) * 64] = st[kb][r] * f;
+    } else {
+        for (int c = c_begin; c + 1 < c_end; c++) chunk(c, std::false_type{});
+        chunk(c_end - 1, std::true_type{});
+    }
+}
+
+// States at the segment ends from the segments' own sums, in place: x_s = exp(A_{e(s-1)} - A_{e(s)}) x_{s-1} + x_s with
+// e(s) the last position of segment s.  One thread per state element; elems = floats per segment, wg_elems = floats per
+// workgroup of the state kernel (whose index modulo BH is the head).
+__global__ __launch_bounds__(256) void scan_segcarry_kernel(ScanArgs a, size_t elems, int wg_elems) {
+    const size_t e = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= elems) return;
+    const int bh = (int)((e / wg_elems) % a.BH);
+    const size_t poff = (size_t)bh * a.NC * GRAN;
+    float run = a.seg_state[e];
+    for (int s = 1; s + 1 < a.nseg; s++) {
+        const int c1 = (s + 1) * a.seg_chunks - 1, c0 = s * a.seg_chunks - 1;   // last chunks of segments s and s - 1
+        const double A1 = (double)a.beta2[poff + GRAN * c1 + GRAN - 1] - a.G2[(size_t)bh * a.NC + c1];
+        const double A0 = (double)a.beta2[poff + GRAN * c0 + GRAN - 1] - a.G2[(size_t)bh * a.NC + c0];
+        run = fast_exp2((float)(A0 - A1)) * run + a.seg_state[(size_t)s * elems + e];
+        a.seg_state[(size_t)s * elems + e] = run;
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -383,10 +433,16 @@ static void launch_state(const ScanArgs& a, hipStream_t st) {
     if constexpr ((D / KS / NW == 32 || D / KS / NW == 64 || D / KS / NW == 128) && NW * KS <= 32) {
         constexpr int lds_bytes = (2 * NW * 32 * 64 + 3 * 2 * GRAN) * 4;
         // (a failure here shows up as a launch error, which the caller reads with hipGetLastError)
-        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&scan_state_kernel<D, KS, NW>),
-                                                           hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        (void)attr;
-        hipLaunchKernelGGL((scan_state_kernel<D, KS, NW>), dim3(a.BH * (D / 32) * KS), dim3(NW * 64), lds_bytes, st, a);
+        (void)lds_limit_once<scan_state_kernel<D, KS, NW, false>>(lds_bytes);
+        const int wgs = a.BH * (D / 32) * KS;
+        if (a.nseg > 1) {
+            (void)lds_limit_once<scan_state_kernel<D, KS, NW, true>>(lds_bytes);
+            hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, true>), dim3(wgs, a.nseg - 1), dim3(NW * 64), lds_bytes, st, a);
+            const size_t elems = (size_t)wgs * NW * (D / KS / NW / 32) * 16 * 64;   // = BH * D * D
+            hipLaunchKernelGGL(scan_segcarry_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st, a, elems,
+                               NW * (D / KS / NW / 32) * 16 * 64);
+        }
+        hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, false>), dim3(wgs, a.nseg), dim3(NW * 64), lds_bytes, st, a);
     }
 }
 
@@ -429,7 +485,29 @@ void scan_plan(int BH, int D, int* KS, int* NW) {
 }
 int scan_key_splits(int BH, int D) { int ks, nw; scan_plan(BH, D, &ks, &nw); return ks; }
 
-int launch_scan(const ScanArgs& a, int KS, hipStream_t st, void (*mark)(int, hipStream_t, bool)) {
+// Segments of a sequence that run side by side: none while heads x value tiles x key ranges fill the chip; otherwise
+// enough for about two workgroups per CU, of at least eight chunks each.
+void scan_segments(int BH, int S, int D, int* nseg, int* seg_chunks) {
+    const int NC = (S + GRAN - 1) / GRAN, wgs = BH * (D / 32) * scan_key_splits(BH, D);
+    int n = 1;
+    if (wgs < 256) {
+        n = (512 + wgs - 1) / wgs;
+        if (n > NC / 8) n = NC / 8;
+        if (n < 1) n = 1;
+    }
+    const int len = (NC + n - 1) / n;
+    *seg_chunks = len;
+    *nseg = (NC + len - 1) / len;
+}
+size_t scan_segment_state_bytes(int BH, int S, int D) {
+    int n, len; scan_segments(BH, S, D, &n, &len);
+    return n > 1 ? (size_t)(n - 1) * BH * D * D * sizeof(float) : 0;
+}
+
+int launch_scan(const ScanArgs& a_in, int KS, hipStream_t st, void (*mark)(int, hipStream_t, bool)) {
+    ScanArgs a = a_in;
+    scan_segments(a.BH, a.S, a.D, &a.nseg, &a.seg_chunks);
+    if (a.nseg > 1 && !a.seg_state) return MLSTM_EWORKSPACE;
     int ks, NW; scan_plan(a.BH, a.D, &ks, &NW);
     if (NW != (a.D / 32 < 4 ? a.D / 32 : 4)) return MLSTM_ESHAPE;
     const int kpw = a.D / KS / NW;

@@ -226,7 +226,7 @@ struct Plan {
     double *G2, *G2r;
     float *alpha2, *beta2, *ek2, *amax2, *m, *alpha2r, *beta2r;
     float *b, *db, *db_rev, *rowdot, *x;
-    float *P, *Nst, *Z, *hpart;
+    float *P, *Nst, *Z, *hpart, *seg_state;
     float *T[8];
     size_t bytes;
 };
@@ -255,6 +255,7 @@ Plan plan_of(char* ws, int BH_, int S_, int D_) {
     const int KS = scan_key_splits(BH_, D_);
     p.hpart = nullptr;
     for (int s = 1; s < KS; s++) { float* t = c.take<float>(N); if (s == 1) p.hpart = t; }
+    p.seg_state = c.take<float>(scan_segment_state_bytes(BH_, S_, D_) / 4);
     for (int t = 0; t < 8; t++) p.T[t] = c.take<float>(N);
     p.bytes = c.off;
     return p;
@@ -284,7 +285,7 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
     if (ge != hipSuccess) return (int)ge;
 
     ScanArgs base{};
-    base.hpart = p.hpart; base.P = p.P; base.Nst = p.Nst; base.M = p.m; base.o = a.o;
+    base.hpart = p.hpart; base.P = p.P; base.Nst = p.Nst; base.M = p.m; base.o = a.o; base.seg_state = p.seg_state;
     base.BH = BH; base.S = S; base.D = D; base.NC = NG;
     auto fwd_gates = [&](ScanArgs& s) { s.alpha2 = p.alpha2; s.beta2 = p.beta2; s.G2 = p.G2; };
     auto rev_gates = [&](ScanArgs& s) { s.alpha2 = p.alpha2r; s.beta2 = p.beta2r; s.G2 = p.G2r; };
