@@ -301,7 +301,7 @@ def main():
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run one plain 256 MiB device copy (torch) before the steps: under rocprofv3 --pmc its "
+                    help="also run a plain 1 GiB device copy (torch), twice, before the steps: under rocprofv3 --pmc its "
                          "FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -314,8 +314,11 @@ def main():
     from _mlstm_pkg import submodule
     ffi = submodule("_ffi")
     if args.calibrate_copy:
-        src = torch.ones(64 * 1024 * 1024, device="cuda:0", dtype=torch.float32)
+        # 1 GiB, copied twice: four times the chip's 256 MB last-level cache, so the second copy's source comes from HBM
+        # (a source that still sits in that cache reads as almost no FETCH_SIZE at all)
+        src = torch.ones(256 * 1024 * 1024, device="cuda:0", dtype=torch.float32)
         dst = torch.empty_like(src)
+        dst.copy_(src)
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
