@@ -18,6 +18,7 @@
 #include "mlstm_device.h"
 #include "mlstm_kernels.h"
 #include <type_traits>
+#include <utility>
 
 namespace mlstm {
 
@@ -30,23 +31,40 @@ __device__ __forceinline__ int perm16(int u) { return (u & ~12) | ((u & 4) << 1)
 template <typename T, int D>
 struct ChunkCfg {
     static constexpr int VW = 128;                                  // value columns per workgroup
-    static constexpr int STAGES = 3;
+    static constexpr int STAGES = 2;                                // LDS stages: the tile worked on and the next one
+    static constexpr int RSETS = 3;                                 // register sets: tiles in flight from memory
     static constexpr size_t K_BYTES = (size_t)GRAN * D * sizeof(T), V_BYTES = (size_t)GRAN * VW * sizeof(T);
     static constexpr size_t TILE_BYTES = STAGES * (K_BYTES + V_BYTES);   // plus one float per position of the chunk
     static constexpr int MAX_L = (int)((160 * 1024 - TILE_BYTES) / (2 * sizeof(float))) / 128 * 128;
 };
 
-// A 16-byte global load issued and waited for by hand, like the direct-to-LDS tile copies next to it (the compiler's
-// own wait counts know nothing of those, and a wait it places for a load of its own would also wait for them)
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void gload16(u32x4& dst, const void* p) { asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(dst) : "v"(p) : "memory"); }
-// wait until at most N of this wave's loads are in flight; the registers pass through so that no use moves above the wait
-template <int N>
-__device__ __forceinline__ void vm_wait(u32x4 (&v)[4]) {
-    asm volatile("s_waitcnt vmcnt(%4)" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]) : "n"(N) : "memory");
+
+// Eight 16-bit elements (four dwords) as floats.  bf16 by hand: one shift or mask per element (the generic vector
+// conversion costs several instructions per element, in a kernel that is bound by instruction issue).
+template <typename T>
+__device__ __forceinline__ void unpack8(const u32x4& d, float (&x)[8]) {
+    if constexpr (std::is_same<T, __bf16>::value) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x[2 * i] = __builtin_bit_cast(float, d[i] << 16);
+            x[2 * i + 1] = __builtin_bit_cast(float, d[i] & 0xffff0000u);
+        }
+    } else {
+        typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+        const h8 v = __builtin_bit_cast(h8, d);
+#pragma unroll
+        for (int e = 0; e < 8; e++) x[e] = (float)v[e];
+    }
 }
 
-template <typename T, int D>
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
+
+// NTT: tiles per chunk as a compile-time constant (the tile loop is then straight-line code), or 0 for any chunk length
+template <typename T, int D, int NTT>
 __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using R = Tr<T>;
@@ -69,7 +87,7 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     if (VH == 2 && (gridDim.x & 15) == 0) { vh = (blockIdx.x >> 3) & 1; pair = (blockIdx.x & 7) | ((blockIdx.x >> 4) << 3); }
     else { vh = blockIdx.x % VH; pair = blockIdx.x / VH; }
     const int cc = pair % a.NCS, bh = pair / a.NCS;
-    const int S = a.S, L = a.L, NT = L / GRAN;
+    const int S = a.S, L = a.L, NT = NTT ? NTT : L / GRAN;
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * a.NG * GRAN, goff = (size_t)bh * a.NG;
     // forward states: sum cc is over chunk cc, relative to its own last position; reverse states (K = Q, V = dH): sum cc
     // is over chunk cc + 1 (the last chunk may be short), relative to the last position of chunk cc
@@ -79,9 +97,6 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     const T* Kh = reinterpret_cast<const T*>(a.K) + a.lk.head(bh) + (size_t)p0 * rsK;
     const T* Vh = reinterpret_cast<const T*>(a.V) + a.lv.head(bh) + (size_t)p0 * rsV + VW * vh;
 
-    TileDma<T, D, GRAN, 256> kdma;   // K tiles by direct loads; every position of a complete chunk exists
-    kdma.init(tid);
-    const auto rk = kdma.rows(tid, (unsigned)(rsK * sizeof(T)));
     SwzTransReader<T, D> krd;        // per-lane offsets of the transposing reads, computed once
     krd.init(lane, (D / 128) * wave);
     SwzTransReader<T, VW> vrd;
@@ -98,84 +113,174 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
 #pragma unroll
             for (int x = 0; x < 16; x++) acc[mb][nb][x] = 0.f;
 
-    // this thread's four 16-byte pieces of a V tile: rows tid/16 + 16 it, piece tid%16; tile j uses register set j % 2
+    // Tiles travel memory -> registers -> LDS.  A thread's pieces of a tile: KP 16-byte pieces of K (piece tid + 256 it of
+    // the tile's rows of CPR pieces) and four of V (rows tid/16 + 16 it, piece tid%16); tile j uses register set j % 3 and
+    // LDS stage j % 2.  Rows past the end of the sequence are clamped (their weights are 0).
+    constexpr int KP = GRAN * ZK::CPR / 256, LPT = KP + 4;   // loads per thread and tile
     const int vrow = tid >> 4, vch = tid & 15;
-    u32x4 vset[2][4];
-    auto issue = [&](auto par_tag, int j) {   // loads of tile j: K into stage j % 3, V into the registers
-        constexpr int P = decltype(par_tag)::value;
-        T* kst = reinterpret_cast<T*>(ks + (j % ST) * Cfg::K_BYTES);
-        if (p0 + GRAN * (j + 1) <= S) kdma.issue(kst, Kh + (size_t)GRAN * j * rsK, rk);
-        else tile_dma<T, D, GRAN, 256>(kst, Kh - (size_t)p0 * rsK, p0 + GRAN * j, S, tid, rsK);   // rows past the end are clamped (their weights are 0)
+    u32x4 kset[Cfg::RSETS][KP], vset[Cfg::RSETS][4];
+    // A thread's pieces lie a fixed number of rows apart (K: 256 / CPR, V: 16): one per-lane element offset each, everything
+    // else of an address is the same for all lanes.  Only the last tile of a short last chunk needs its rows clamped.
+    constexpr int KROWS = 256 / ZK::CPR;
+    const unsigned koff = (unsigned)((tid / ZK::CPR) * rsK + 8 * (tid % ZK::CPR)), voff = (unsigned)(vrow * rsV + 8 * vch);
+    auto issue = [&](auto set_tag, int j) __attribute__((always_inline)) {
+        constexpr int P = decltype(set_tag)::value;
+        if (p0 + GRAN * (j + 1) <= S) {
+            const T* kt = Kh + (size_t)GRAN * j * rsK;
+            const T* vt = Vh + (size_t)GRAN * j * rsV;
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
-            int pos = GRAN * j + vrow + 16 * it;
-            pos = p0 + pos < S ? pos : S - 1 - p0;
-            gload16(vset[P][it], Vh + (size_t)pos * rsV + 8 * vch);
+            for (int it = 0; it < KP; it++) kset[P][it] = *reinterpret_cast<const u32x4*>(kt + (size_t)(KROWS * it) * rsK + koff);
+#pragma unroll
+            for (int it = 0; it < 4; it++) vset[P][it] = *reinterpret_cast<const u32x4*>(vt + (size_t)(16 * it) * rsV + voff);
+        } else {
+#pragma unroll
+            for (int it = 0; it < KP; it++) {
+                const int pc = tid + 256 * it;
+                int pos = GRAN * j + pc / ZK::CPR;
+                pos = p0 + pos < S ? pos : S - 1 - p0;
+                kset[P][it] = *reinterpret_cast<const u32x4*>(Kh + (size_t)pos * rsK + 8 * (pc % ZK::CPR));
+            }
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                int pos = GRAN * j + vrow + 16 * it;
+                pos = p0 + pos < S ? pos : S - 1 - p0;
+                vset[P][it] = *reinterpret_cast<const u32x4*>(Vh + (size_t)pos * rsV + 8 * vch);
+            }
         }
+        __builtin_amdgcn_sched_barrier(0);   // the loads go out here, not where the scheduler would like them
     };
-    auto commit = [&](auto par_tag, int j) {  // V of tile j, times the positions' weights, into stage j % 3
-        constexpr int P = decltype(par_tag)::value;
+    // K of tile j as it is, V times the positions' weights, into stage j % 2; in four parts (one per contraction step of the
+    // tile that is being worked on meanwhile), part < 0: all of it
+    auto commit = [&](auto set_tag, int j, int part) __attribute__((always_inline)) {
+        constexpr int P = decltype(set_tag)::value;
         typedef typename R::vec4 V4;
         struct Pair { V4 lo, hi; };
 #pragma unroll
+        for (int it = 0; it < KP; it++) {
+            if (part >= 0 && it / (KP / 4) != part) continue;
+            const int pc = tid + 256 * it;
+            *reinterpret_cast<u32x4*>(ks + (j % ST) * Cfg::K_BYTES + ZK::off(pc / ZK::CPR, 8 * (pc % ZK::CPR))) = kset[P][it];
+        }
+#pragma unroll
         for (int it = 0; it < 4; it++) {
+            if (part >= 0 && it != part) continue;
             const int row = vrow + 16 * it;
             const float w = sw[GRAN * j + row];
-            const Pair in = __builtin_bit_cast(Pair, vset[P][it]);
+            float x[8];
+            unpack8<T>(vset[P][it], x);
             Pair out;
-            out.lo = R::cvt4(__builtin_convertvector(in.lo, f32x4) * w);
-            out.hi = R::cvt4(__builtin_convertvector(in.hi, f32x4) * w);
+            out.lo = R::cvt4(f32x4{x[0] * w, x[1] * w, x[2] * w, x[3] * w});
+            out.hi = R::cvt4(f32x4{x[4] * w, x[5] * w, x[6] * w, x[7] * w});
             *reinterpret_cast<Pair*>(vs + (j % ST) * Cfg::V_BYTES + ZV::off(row, 8 * vch)) = out;
         }
     };
-    auto compute = [&](int t) {
+    auto compute = [&](int t, auto&& hook) __attribute__((always_inline)) {
         const T* kt = reinterpret_cast<const T*>(ks + (t % ST) * Cfg::K_BYTES);
         const T* vt = reinterpret_cast<const T*>(vs + (t % ST) * Cfg::V_BYTES);
+        // the operand reads of a contraction step run one step ahead of its MFMAs (read, wait, multiply in turns left the
+        // matrix unit idle for an LDS round trip per step: 3000 cycles per tile for 1024 of MFMAs, measured)
+        constexpr int NSTEP = GRAN / KW;
+        frag af[2][MB], bf[2][NB];
+        auto rd = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
-        for (int s = 0; s < GRAN / KW; s++) {
-            frag af[MB], bf[NB];
+            for (int mb = 0; mb < MB; mb++) af[s & 1][mb] = krd.read(kt, KW * s, mb);
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) af[mb] = krd.read(kt, KW * s, mb);
+            for (int nb = 0; nb < NB; nb++) bf[s & 1][nb] = vrd.read(vt, KW * s, nb);
+        };
+        rd(0);
 #pragma unroll
-            for (int nb = 0; nb < NB; nb++) bf[nb] = vrd.read(vt, KW * s, nb);
+        for (int s = 0; s < NSTEP; s++) {
+            if (s + 1 < NSTEP) rd(s + 1);
+            hook(s);
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                for (int nb = 0; nb < NB; nb++) R::mma(acc[mb][nb], af[mb], bf[nb]);
+                for (int nb = 0; nb < NB; nb++) R::mma(acc[mb][nb], af[s & 1][mb], bf[s & 1][nb]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         if (vh == 0) {   // the vector state's share of this tile
             const char* kb = reinterpret_cast<const char*>(kt);
 #pragma unroll
             for (int j = 0; j < PPT; j++) {
                 const int pos = PPT * pg + j;
-                const f32x8 kv = __builtin_convertvector(*reinterpret_cast<const frag*>(kb + ZK::off(pos, 8 * kc)), f32x8);
-                nacc += kv * sw2[GRAN * t + pos];
+                float x[8];
+                unpack8<T>(*reinterpret_cast<const u32x4*>(kb + ZK::off(pos, 8 * kc)), x);
+                const float w2 = sw2[GRAN * t + pos];
+#pragma unroll
+                for (int e = 0; e < 8; e++) nacc[e] += x[e] * w2;
             }
         }
     };
-    // Iteration t: V of tile t + 1 (loaded during the previous iteration) moves from registers to LDS, the loads of tile
-    // t + 2 are issued, tile t is worked on.  The wait is for ALL of the wave's loads: a counted wait (vmcnt(n) with the
-    // n loads just issued still in flight) was tried, with the loads of tile t + 2 issued first, and gave wrong states
-    // now and then -- direct-to-LDS loads and loads into registers evidently do not retire in one common order.
-    auto iteration = [&](auto par_tag, int t) {
-        constexpr int P = decltype(par_tag)::value;   // t % 2
-        if (t >= 1 && t + 1 < NT) {
-            vm_wait<0>(vset[P ^ 1]);   // tile t + 1 has landed (K: this wave's share)
-            commit(std::integral_constant<int, P ^ 1>{}, t + 1);
-        }
-        if (t + 2 < NT) issue(std::integral_constant<int, P>{}, t + 2);
-        compute(t);
+    // Iteration t (register set P = t % 3): the loads of tile t + 3 go out into the registers tile t left in the previous
+    // iteration; tile t is worked on, and between its MFMAs tile t + 1 moves to the LDS stage that tile t - 1 left behind the
+    // last barrier.  Two to three tiles are in flight while a tile is worked on.  The loads are ordinary ones, so that the compiler places the counted
+    // waits itself; it counts exactly in straight-line code (hence NTT: the default chunk's eight iterations are unrolled)
+    // and falls back to waiting for everything across a loop's back edge.  Loads issued by hand -- direct-to-LDS copies of
+    // K, or register loads from inline assembly -- gave wrong states now and then at full size as soon as a wait was a
+    // counted one: the compiler moves or stashes a register it believes written while the load is still in flight.  With
+    // one tile in flight and a wait for everything the kernel waited for memory latency in every iteration.
+    auto iteration = [&](auto set_tag, int t) __attribute__((always_inline)) {
+        constexpr int P = decltype(set_tag)::value, P1 = (P + 1) % 3;
+        if (t + 3 < NT) issue(std::integral_constant<int, P>{}, t + 3);
+        // (the vector work and LDS writes of the hand-over ride between the MFMAs: done in one piece before them they
+        // cost 1200 cycles per tile next to 1024 of MFMAs, measured)
+        compute(t, [&](int s) __attribute__((always_inline)) { if (t + 1 < NT) commit(std::integral_constant<int, P1>{}, t + 1, s); });
         __syncthreads();
     };
 
-    issue(std::integral_constant<int, 0>{}, 0);
-    issue(std::integral_constant<int, 1>{}, 1);
-    {   // the positions' weights.  Forward: w_j = exp(a_j - A_e) / sqrt(D) for both sums, e the chunk's last position.
-        // Reverse: rho_i = exp(A_e - A_i) / sqrt(D), e the last position BEFORE the chunk, times 1/n_i (matrix sum) or db_i
-        // (vector sum), the per-row scalars of the dQ pass.
+    // The positions' weights.  Forward: w_j = exp(a_j - A_e) / sqrt(D) for both sums, e the chunk's last position.
+    // Reverse: rho_i = exp(A_e - A_i) / sqrt(D), e the last position BEFORE the chunk, times 1/n_i (matrix sum) or db_i
+    // (vector sum), the per-row scalars of the dQ pass.
+    const float log2scale = -0.5f * __log2f((float)D);
+    if constexpr (NTT > 0) {
+        // Their inputs are requested first and used behind the first tile's loads: the waits the compiler places for them
+        // then count the tile loads as "behind" and do not wait for those (requested after the tiles, the weights waited
+        // for all three tiles: 13 k cycles before the first iteration, measured).  The other two tiles' loads follow one
+        // by one, so that the first tile's data is not queued behind theirs.
+        constexpr int WPT = NTT * GRAN / 256;   // positions per thread
+        float x0[WPT], x1[WPT], x2[WPT];
+        double xg[WPT];
         const float bend = a.beta2[poff + pe];
         const double Gend = a.G2[goff + pe / GRAN];
-        const float log2scale = -0.5f * __log2f((float)D);
+#pragma unroll
+        for (int n = 0; n < WPT; n++) {
+            int pos = p0 + tid + 256 * n;
+            pos = pos < S ? pos : S - 1;
+            xg[n] = a.G2[goff + pos / GRAN];
+            if (a.reverse) { x0[n] = a.beta2[poff + pos]; x1[n] = a.inv_n[poff + pos]; x2[n] = a.db[poff + pos]; }
+            else { x0[n] = a.alpha2[poff + pos]; x1[n] = 0.f; x2[n] = 0.f; }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue(std::integral_constant<int, 0>{}, 0);
+#pragma unroll
+        for (int n = 0; n < WPT; n++) {
+            const int p = tid + 256 * n;
+            float w = 0.f, w2 = 0.f;
+            if (p0 + p < S) {
+                if (a.reverse) {
+                    const float rho = fast_exp2(bend - x0[n] + (float)(xg[n] - Gend) + log2scale);
+                    w = rho * x1[n];
+                    w2 = rho * x2[n];
+                } else {
+                    w = w2 = fast_exp2(x0[n] - bend + (float)(Gend - xg[n]) + log2scale);
+                }
+            }
+            sw[p] = w;
+            sw2[p] = w2;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        issue(std::integral_constant<int, 1>{}, 1);   // (NT >= 2: a chunk is a multiple of 128 positions)
+        __syncthreads();   // the weights are in LDS
+        commit(std::integral_constant<int, 0>{}, 0, -1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
+        __syncthreads();
+    } else {
+        issue(std::integral_constant<int, 0>{}, 0);
+        issue(std::integral_constant<int, 1>{}, 1);
+        if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
+        const float bend = a.beta2[poff + pe];
+        const double Gend = a.G2[goff + pe / GRAN];
         for (int p = tid; p < L; p += 256) {
             const int pos = p0 + p;
             float w = 0.f, w2 = 0.f;
@@ -191,16 +296,18 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
             sw[p] = w;
             sw2[p] = w2;
         }
+        __syncthreads();   // the weights are in LDS
+        commit(std::integral_constant<int, 0>{}, 0, -1);
+        __syncthreads();
     }
-    vm_wait<0>(vset[0]);
-    vm_wait<0>(vset[1]);
-    __syncthreads();
-    commit(std::integral_constant<int, 0>{}, 0);
-    commit(std::integral_constant<int, 1>{}, 1);
-    __syncthreads();
-    for (int t = 0; t < NT; t += 2) {   // (L is a multiple of 128: an even number of tiles)
-        iteration(std::integral_constant<int, 0>{}, t);
-        iteration(std::integral_constant<int, 1>{}, t + 1);
+    if constexpr (NTT > 0) {
+        static_for<NTT>([&](auto tt) __attribute__((always_inline)) { iteration(std::integral_constant<int, decltype(tt)::value % 3>{}, decltype(tt)::value); });
+    } else {
+        for (int t = 0; t < NT; t += 3) {
+            iteration(std::integral_constant<int, 0>{}, t);
+            if (t + 1 < NT) iteration(std::integral_constant<int, 1>{}, t + 1);
+            if (t + 2 < NT) iteration(std::integral_constant<int, 2>{}, t + 2);
+        }
     }
     // accumulator block (mb, nb): column (value) 32 nb + c32, rows (keys) 8 (r / 4) + 4 h + r % 4
     float* out = a.dC + ((size_t)bh * a.NCS + cc) * D * D + VW * vh;
@@ -333,10 +440,16 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
 template <typename T, int D>
 static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     using Cfg = ChunkCfg<T, D>;
-    auto kern = chunk_sum_kernel<T, D>;
-    if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D>>(160 * 1024); e != hipSuccess) return (int)e;
     if (a.L > Cfg::MAX_L) return MLSTM_ESHAPE;
-    hipLaunchKernelGGL(kern, dim3(a.BH * a.NCS * (D / Cfg::VW)), dim3(256), Cfg::TILE_BYTES + 2 * (size_t)a.L * sizeof(float), st, a);
+    const dim3 grid(a.BH * a.NCS * (D / Cfg::VW));
+    const size_t lds = Cfg::TILE_BYTES + 2 * (size_t)a.L * sizeof(float);
+    if (a.L == 8 * GRAN) {   // the default chunk length
+        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 8>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 8>), grid, dim3(256), lds, st, a);
+    } else {
+        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 0>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 0>), grid, dim3(256), lds, st, a);
+    }
     // one carry kernel: the value-major one writes both layouts and the vector states
     if (a.CstT) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D>), dim3((D / 64) * (D / 64), a.BH), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((chunk_carry_kernel<T, D>), dim3(D * D / 8 / 256, a.BH), dim3(256), 0, st, a);
