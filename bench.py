@@ -334,6 +334,7 @@ def main():
         few = max(min(args.steps, 20), 5)
         out["secondary"] = [run_matmul(ffi, args.workload, few, 3, precise=True, host=host)[0],
                             run_matmul(ffi, "cfg5_B2_H32_S16384_D128_bf16", few, 3)[0],
+                            run_matmul(ffi, "cfg2_B1_H4_S2048_D64_f32", max(args.steps // 4, 10), 3)[0],
                             run_scan(ffi, max(args.steps, 20), 5), run_scan(ffi, max(args.steps // 4, 10), 3, backward=True)]
     if not args.no_cpu_baseline:
         S, D = WORKLOADS[args.workload][2:4]
