@@ -8,8 +8,8 @@ Prints ONE JSON line.  `value` is algorithmic TFLOP/s: 7*D*S*(S+1) useful (causa
 than that, which `executed_tflops` / `executed_frac` report beside it.  `roofline` is the dominant kernel (the
 column-parallel backward tile kernel) timed with HIP events on its launch stream during the timed steps;
 `cpu_baseline` times the C restatement of the reference's CPU path, `cpu_baseline_torch` the dense PyTorch formulas, on
-the same seeded inputs; `secondary` holds the other workloads (long context, scan form, split mode), each measured the
-same way with a roofline object of its own.
+the same seeded inputs; `secondary` holds the other workloads (long context, scan form, split mode, sLSTM cell), each measured the
+same way (the tile and scan workloads with a roofline object of their own).
 """
 import argparse
 import hashlib
@@ -291,12 +291,68 @@ def run_scan(ffi, steps, warmup, backward=False, shape=(1, 4, 2048, 1024), tag="
     }
 
 
+def run_slstm(ffi, steps, warmup, shape=(16, 4, 2048, 64)):
+    """sLSTM cell, forward (keeping the state for the backward) + backward, fp32.  The recurrence through h is sequential in
+    t: one workgroup per (batch, head) walks the sequence, so what is measured is the time of one step of that walk."""
+    L = ffi.lib()
+    B, NH, S, DH = shape
+    wl = f"slstm_B{B}_NH{NH}_S{S}_DH{DH}_f32"
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    wx = torch.randn((B, S, 4, NH, DH), generator=g).to(dev)
+    r = (torch.randn((NH, 4, DH, DH), generator=g) * DH ** -0.5).to(dev)
+    b = (torch.randn((NH, 4, DH), generator=g) * 0.1).to(dev)
+    dh = torch.randn((B, S, NH, DH), generator=g).to(dev)
+    h = torch.empty_like(dh)
+    saved = torch.empty(int(L.slstm_saved_bytes(B, NH, S, DH)), dtype=torch.uint8, device=dev)
+    ws_n = int(L.slstm_workspace_bytes(B, NH, S, DH))
+    ws = torch.empty(ws_n, dtype=torch.uint8, device=dev)
+    dwx, dr, db = torch.empty_like(wx), torch.empty_like(r), torch.empty_like(b)
+    st, P = ffi.stream_ptr(), ffi.ptr
+
+    def fwd():
+        ffi.check_rc(L.slstm_forward_ex(P(wx), P(r), P(b), P(h), P(saved), B, NH, S, DH, 1, st), "slstm_forward_ex")
+
+    def bwd():
+        ffi.check_rc(L.slstm_backward_ex(P(dh), P(h), P(r), P(saved), P(dwx), P(dr), P(db), B, NH, S, DH, 1, P(ws), ws_n, st),
+                     "slstm_backward_ex")
+
+    for _ in range(warmup):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fwd(); bwd()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(3)]   # (the calls run on torch's current stream)
+    f_ms = b_ms = 0.0
+    for _ in range(max(steps // 4, 1)):
+        ev[0].record(); fwd(); ev[1].record(); bwd(); ev[2].record()
+        torch.cuda.synchronize()
+        f_ms += ev[0].elapsed_time(ev[1]); b_ms += ev[1].elapsed_time(ev[2])
+    f_ms /= max(steps // 4, 1); b_ms /= max(steps // 4, 1)
+    ms_step = (t1 - t0) * 1e3 / steps
+    # wx in, h and the seven kept values out; those and dh in, dwx out; dwx and h in again for dR and db
+    bytes_compulsory = 29.0 * B * S * NH * DH * 4
+    return {
+        "metric": "sLSTM cell forward+backward, sequence positions per second, " + wl,
+        "value": B * S / (ms_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic", "config": {"workload": wl, "B": B, "NH": NH, "S": S, "DH": DH, "forget": "sigmoid"},
+        "forward_ms": f_ms, "backward_ms": b_ms,
+        # the quantity the kernels are built around: wall time per step of the recurrence (B * NH walks side by side)
+        "ns_per_recurrence_step": {"forward": f_ms * 1e6 / S, "backward": b_ms * 1e6 / S},
+        "hbm_gbs": bytes_compulsory / (ms_step * 1e-3) / 1e9, "hbm_frac": bytes_compulsory / (ms_step * 1e-3) / 8e12,
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
-    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan", "cfg3_scan_backward", "long_scan"])
+    ap.add_argument("--workload", default="cfg4_B4_H8_S4096_D256_bf16", choices=sorted(WORKLOADS) + ["cfg3_scan", "cfg3_scan_backward", "long_scan", "slstm"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
@@ -325,6 +381,9 @@ def main():
     if args.workload == "long_scan":   # one long sequence: the state walk runs in segments side by side
         print(json.dumps(run_scan(ffi, args.steps, args.warmup, shape=(1, 1, 65536, 128), tag="long")))
         return
+    if args.workload == "slstm":
+        print(json.dumps(run_slstm(ffi, args.steps, args.warmup)))
+        return
     if args.workload in ("cfg3_scan", "cfg3_scan_backward"):
         print(json.dumps(run_scan(ffi, args.steps, args.warmup, backward=args.workload.endswith("backward"))))
         return
@@ -335,7 +394,8 @@ def main():
         out["secondary"] = [run_matmul(ffi, args.workload, few, 3, precise=True, host=host)[0],
                             run_matmul(ffi, "cfg5_B2_H32_S16384_D128_bf16", few, 3)[0],
                             run_matmul(ffi, "cfg2_B1_H4_S2048_D64_f32", max(args.steps // 4, 10), 3)[0],
-                            run_scan(ffi, max(args.steps, 20), 5), run_scan(ffi, max(args.steps // 4, 10), 3, backward=True)]
+                            run_scan(ffi, max(args.steps, 20), 5), run_scan(ffi, max(args.steps // 4, 10), 3, backward=True),
+                            run_slstm(ffi, max(args.steps // 4, 10), 3)]
     if not args.no_cpu_baseline:
         S, D = WORKLOADS[args.workload][2:4]
         out["cpu_baseline"] = cpu_baseline(host, S, D)

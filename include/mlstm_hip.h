@@ -222,6 +222,27 @@ int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, c
                            const void* o, void* dq, void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S,
                            int D, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * sLSTM cell, forward and backward (fp32).  The reference lists the cell as an open item (README.md:9) and has no code
+ * for it; these implement the published cell (Beck et al., arXiv:2405.04517, section 2.2 and appendix A.2) per head:
+ *   pre_g = wx[b,t,g,h,:] + r[h,g] h_{t-1} + b[h,g]   (g = i, f, z, o),  m_t = max(log f_t + m_{t-1}, i~),
+ *   c_t = exp(log f_t + m_{t-1} - m_t) c_{t-1} + exp(i~ - m_t) tanh(z~),  n_t likewise with 1,  h_t = sigmoid(o~) c_t / n_t,
+ * log f_t = f~ or, with forget_sigmoid != 0, logsigmoid(f~); zero initial state.
+ * wx, dwx: [B,S,4,NH,DH] (the input projections of the four gates, computed by the caller's GEMM); r, dr: [NH,4,DH,DH]
+ * (r[h][g][j][k]: unit j from unit k); b, db: [NH,4,DH]; h, dh: [B,S,NH,DH]; DH in {32, 64, 128}.
+ * slstm_forward_ex writes what the backward needs into `saved` (slstm_saved_bytes; may be NULL for inference; opaque:
+ * written and read by the same build of the library).  All tensors dense.
+ * slstm_backward_ex needs a workspace of slstm_workspace_bytes.  One workgroup per (batch, head) walks the sequence:
+ * the cell is sequential in t by construction.
+ */
+size_t slstm_saved_bytes(int B, int NH, int S, int DH);
+size_t slstm_workspace_bytes(int B, int NH, int S, int DH);
+int slstm_forward_ex(const float* wx, const float* r, const float* b, float* h, float* saved, int B, int NH, int S, int DH,
+                     int forget_sigmoid, void* stream);
+int slstm_backward_ex(const float* dh, const float* h, const float* r, const float* saved, float* dwx, float* dr, float* db,
+                      int B, int NH, int S, int DH, int forget_sigmoid, void* workspace, size_t workspace_bytes,
+                      void* stream);
+
 /* Bytes of scratch the operation needs for this shape (the torch.zeros workspaces of mlstm_scan.py:299-307 and
  * the db buffer of mlstm_matmul.py:394 are the reference's counterparts). */
 size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype);

@@ -42,7 +42,7 @@ def test_oracle_reproduces_scan_golden():
 def test_library_exports_every_declared_symbol():
     ffi = submodule("_ffi")
     header = open(os.path.join(ROOT, "include", "mlstm_hip.h")).read()
-    declared = set(re.findall(r"^(?:int|size_t|const char\*)\s+(mlstm_\w+)\s*\(", header, flags=re.M))
+    declared = set(re.findall(r"^(?:int|size_t|const char\*)\s+((?:mlstm|slstm)_\w+)\s*\(", header, flags=re.M))
     assert declared == set(ffi.exported_symbols()), declared ^ set(ffi.exported_symbols())
     L = ffi.lib()
     for sym in declared:

@@ -71,6 +71,15 @@ def lib():
         L.mlstm_forward_save_lx.argtypes = [vp] * 9 + [sz] + [ci] * 6 + [lp, vp, sz, vp]
         L.mlstm_backward_saved_lx.restype = ci
         L.mlstm_backward_saved_lx.argtypes = [vp] * 10 + [sz] + [vp] * 5 + [ci] * 6 + [lp, vp, sz, vp]
+        fp = ctypes.c_void_p
+        L.slstm_saved_bytes.restype = sz
+        L.slstm_saved_bytes.argtypes = [ci] * 4
+        L.slstm_workspace_bytes.restype = sz
+        L.slstm_workspace_bytes.argtypes = [ci] * 4
+        L.slstm_forward_ex.restype = ci
+        L.slstm_forward_ex.argtypes = [fp] * 5 + [ci] * 5 + [vp]
+        L.slstm_backward_ex.restype = ci
+        L.slstm_backward_ex.argtypes = [fp] * 7 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_scan_forward_ex.restype = ci
         L.mlstm_scan_forward_ex.argtypes = [vp] * 7 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_scan_backward_ex.restype = ci
@@ -97,7 +106,7 @@ def lib():
 
 def exported_symbols():
     return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
-            "mlstm_scan_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
+            "mlstm_scan_backward_ex", "slstm_saved_bytes", "slstm_workspace_bytes", "slstm_forward_ex", "slstm_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
