@@ -37,10 +37,11 @@ CSRC = os.path.join(ROOT, "xlstm-triton-cuda-implementation_amd", "csrc")
 
 
 def kernel_source_hash():
-    """Identifies the kernels a measured traffic figure belongs to: sha256 over the device sources."""
+    """Identifies the kernels a measured traffic figure belongs to: sha256 over the device sources of the mLSTM kernels
+    (mlstm_*.hip and the headers they share; the sLSTM cell is a file of its own that none of them includes)."""
     hsh = hashlib.sha256()
     for name in sorted(os.listdir(CSRC)):
-        if name.endswith((".hip", ".h")):
+        if name.startswith("mlstm_") and name.endswith((".hip", ".h")):
             hsh.update(name.encode())
             hsh.update(open(os.path.join(CSRC, name), "rb").read())
     return hsh.hexdigest()[:16]
