@@ -11,7 +11,7 @@
 //   chunk_sum_kernel    per (head, chunk, 128 value columns): dC_c = sum_{j in chunk} w_j k_j v_j^T with
 //                       w_j = exp(a_j - A_{e_c}) / sqrt(D), as a bf16 / fp16 MFMA product over the chunk's positions (both
 //                       operands are contracted over positions: transposing LDS reads; V is scaled by w on its way
-//                       into LDS), fp32 result; and dn_c = sum_j w_j k_j.
+//                       into LDS), fp32 result; and dn_c = sum_j w_j k_j.  Eight waves: four multiply, four bring the tiles.
 //   chunk_carry_kernel  C~_c = gamma_c C~_{c-1} + dC_c over the chunks of a head (gamma_c = exp(A_{e_{c-1}} - A_{e_c})),
 //                       element-wise, written in the element type; n~_c likewise, in place, fp32.
 // State rows are stored in the order in which the row kernel's second product contracts them (see PERM16 below).
@@ -65,7 +65,7 @@ __device__ __forceinline__ void static_for(F&& f) { static_for_impl(std::make_in
 
 // NTT: tiles per chunk as a compile-time constant (the tile loop is then straight-line code), or 0 for any chunk length
 template <typename T, int D, int NTT>
-__global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
+__global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using R = Tr<T>;
     using Cfg = ChunkCfg<T, D>;
@@ -80,7 +80,12 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     float* const sw = reinterpret_cast<float*>(smem + Cfg::TILE_BYTES);   // [L] position weights of the matrix sum
     float* const sw2 = sw + a.L;                                           // [L] ... of the vector sum
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
+    // Eight waves, two on every SIMD.  Waves 0..3 multiply: operand reads and MFMAs, nothing else.  Waves 4..7 feed them: they
+    // load the tiles, scale V, write the LDS stages and add up the vector state from the K pieces they hold anyway.  With
+    // four waves doing both in turn the kernel was bound by instruction issue (about 430 other instructions per tile next to
+    // 1024 cycles of MFMAs, on a SIMD with nothing else to run); the two kinds of work now overlap.
+    const bool feeder = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) != 0;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
     // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own: the VH workgroups of a (head, chunk), which read
     // the same K, sit 8 apart in the launch order, on one XCD
     int vh, pair;
@@ -97,22 +102,14 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
     const T* Kh = reinterpret_cast<const T*>(a.K) + a.lk.head(bh) + (size_t)p0 * rsK;
     const T* Vh = reinterpret_cast<const T*>(a.V) + a.lv.head(bh) + (size_t)p0 * rsV + VW * vh;
 
-    SwzTransReader<T, D> krd;        // per-lane offsets of the transposing reads, computed once
-    krd.init(lane, (D / 128) * wave);
-    SwzTransReader<T, VW> vrd;
-    vrd.init(lane, 0);
-    // vector state: thread (pg, kc) adds positions PPT pg .. of every tile for the eight keys 8 kc .. 8 kc + 7
+    // vector state: a feeder thread's K pieces of a tile are rows pg + NPG it (it < KP) of the eight keys 8 kc .. 8 kc + 7
     const int kc = tid & (D / 8 - 1), pg = tid / (D / 8);
-    constexpr int NPG = 256 / (D / 8), PPT = GRAN / NPG;
-    f32x8 nacc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    f32x16 acc[MB][NB];
-#pragma unroll
-    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-        for (int nb = 0; nb < NB; nb++)
-#pragma unroll
-            for (int x = 0; x < 16; x++) acc[mb][nb][x] = 0.f;
+    constexpr int NPG = 256 / (D / 8);
 
+    // The two kinds of waves run code of their own from here on (every value of one kind is dead in the other: the registers
+    // of a wave hold either the accumulators or the tiles in flight); both pass the same barriers.
+    auto feed = [&]() __attribute__((always_inline)) {
+    f32x8 nacc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     // Tiles travel memory -> registers -> LDS.  A thread's pieces of a tile: KP 16-byte pieces of K (piece tid + 256 it of
     // the tile's rows of CPR pieces) and four of V (rows tid/16 + 16 it, piece tid%16); tile j uses register set j % 3 and
     // LDS stage j % 2.  Rows past the end of the sequence are clamped (their weights are 0).
@@ -149,21 +146,25 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
         }
         __builtin_amdgcn_sched_barrier(0);   // the loads go out here, not where the scheduler would like them
     };
-    // K of tile j as it is, V times the positions' weights, into stage j % 2; in four parts (one per contraction step of the
-    // tile that is being worked on meanwhile), part < 0: all of it
-    auto commit = [&](auto set_tag, int j, int part) __attribute__((always_inline)) {
+    // K of tile j as it is, V times the positions' weights, into stage j % 2
+    auto commit = [&](auto set_tag, int j) __attribute__((always_inline)) {
         constexpr int P = decltype(set_tag)::value;
         typedef typename R::vec4 V4;
         struct Pair { V4 lo, hi; };
 #pragma unroll
         for (int it = 0; it < KP; it++) {
-            if (part >= 0 && it / (KP / 4) != part) continue;
             const int pc = tid + 256 * it;
             *reinterpret_cast<u32x4*>(ks + (j % ST) * Cfg::K_BYTES + ZK::off(pc / ZK::CPR, 8 * (pc % ZK::CPR))) = kset[P][it];
+            if (vh == 0) {   // the vector state's share of this piece
+                float x[8];
+                unpack8<T>(kset[P][it], x);
+                const float w2 = sw2[GRAN * j + pc / ZK::CPR];
+#pragma unroll
+                for (int e = 0; e < 8; e++) nacc[e] += x[e] * w2;
+            }
         }
 #pragma unroll
         for (int it = 0; it < 4; it++) {
-            if (part >= 0 && it != part) continue;
             const int row = vrow + 16 * it;
             const float w = sw[GRAN * j + row];
             float x[8];
@@ -174,7 +175,132 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
             *reinterpret_cast<Pair*>(vs + (j % ST) * Cfg::V_BYTES + ZV::off(row, 8 * vch)) = out;
         }
     };
-    auto compute = [&](int t, auto&& hook) __attribute__((always_inline)) {
+    // Iteration t, feeders (register set P = t % 3): the loads of tile t + 3 go out into the registers tile t left in the previous
+    // iteration; tile t + 1 moves to the LDS stage that tile t - 1 left behind the last barrier.  The others multiply tile t.
+    // Two to three tiles are in flight while a tile is worked on.  The loads are ordinary ones, so that the compiler places the counted
+    // waits itself; it counts exactly in straight-line code (hence NTT: the default chunk's eight iterations are unrolled)
+    // and falls back to waiting for everything across a loop's back edge.  Loads issued by hand -- direct-to-LDS copies of
+    // K, or register loads from inline assembly -- gave wrong states now and then at full size as soon as a wait was a
+    // counted one: the compiler moves or stashes a register it believes written while the load is still in flight.  With
+    // one tile in flight and a wait for everything the kernel waited for memory latency in every iteration.
+    auto iteration = [&](auto set_tag, int t) __attribute__((always_inline)) {
+        constexpr int P = decltype(set_tag)::value, P1 = (P + 1) % 3;
+        if (t + 3 < NT) issue(std::integral_constant<int, P>{}, t + 3);
+        if (t + 1 < NT) commit(std::integral_constant<int, P1>{}, t + 1);
+        __syncthreads();
+    };
+
+    // The positions' weights.  Forward: w_j = exp(a_j - A_e) / sqrt(D) for both sums, e the chunk's last position.
+    // Reverse: rho_i = exp(A_e - A_i) / sqrt(D), e the last position BEFORE the chunk, times 1/n_i (matrix sum) or db_i
+    // (vector sum), the per-row scalars of the dQ pass.
+    const float log2scale = -0.5f * __log2f((float)D);
+    if constexpr (NTT > 0) {
+        // Their inputs are requested first and used behind the first tile's loads: the waits the compiler places for them
+        // then count the tile loads as "behind" and do not wait for those (requested after the tiles, the weights waited
+        // for all three tiles: 13 k cycles before the first iteration, measured).  The other two tiles' loads follow one
+        // by one, so that the first tile's data is not queued behind theirs.
+        {
+            constexpr int WPT = NTT * GRAN / 256;   // positions per thread
+            float x0[WPT], x1[WPT], x2[WPT];
+            double xg[WPT];
+            const float bend = a.beta2[poff + pe];
+            const double Gend = a.G2[goff + pe / GRAN];
+#pragma unroll
+            for (int n = 0; n < WPT; n++) {
+                int pos = p0 + tid + 256 * n;
+                pos = pos < S ? pos : S - 1;
+                xg[n] = a.G2[goff + pos / GRAN];
+                if (a.reverse) { x0[n] = a.beta2[poff + pos]; x1[n] = a.inv_n[poff + pos]; x2[n] = a.db[poff + pos]; }
+                else { x0[n] = a.alpha2[poff + pos]; x1[n] = 0.f; x2[n] = 0.f; }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            issue(std::integral_constant<int, 0>{}, 0);
+#pragma unroll
+            for (int n = 0; n < WPT; n++) {
+                const int p = tid + 256 * n;
+                float w = 0.f, w2 = 0.f;
+                if (p0 + p < S) {
+                    if (a.reverse) {
+                        const float rho = fast_exp2(bend - x0[n] + (float)(xg[n] - Gend) + log2scale);
+                        w = rho * x1[n];
+                        w2 = rho * x2[n];
+                    } else {
+                        w = w2 = fast_exp2(x0[n] - bend + (float)(Gend - xg[n]) + log2scale);
+                    }
+                }
+                sw[p] = w;
+                sw2[p] = w2;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            issue(std::integral_constant<int, 1>{}, 1);   // (NT >= 2: a chunk is a multiple of 128 positions)
+        }
+        __syncthreads();   // the weights are in LDS
+        commit(std::integral_constant<int, 0>{}, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
+        __syncthreads();
+    } else {
+        {
+            issue(std::integral_constant<int, 0>{}, 0);
+            issue(std::integral_constant<int, 1>{}, 1);
+            if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
+            const float bend = a.beta2[poff + pe];
+            const double Gend = a.G2[goff + pe / GRAN];
+            for (int p = tid; p < L; p += 256) {
+                const int pos = p0 + p;
+                float w = 0.f, w2 = 0.f;
+                if (pos < S) {
+                    if (a.reverse) {
+                        const float rho = fast_exp2(bend - a.beta2[poff + pos] + (float)(a.G2[goff + pos / GRAN] - Gend) + log2scale);
+                        w = rho * a.inv_n[poff + pos];
+                        w2 = rho * a.db[poff + pos];
+                    } else {
+                        w = w2 = fast_exp2(a.alpha2[poff + pos] - bend + (float)(Gend - a.G2[goff + pos / GRAN]) + log2scale);
+                    }
+                }
+                sw[p] = w;
+                sw2[p] = w2;
+            }
+        }
+        __syncthreads();   // the weights are in LDS
+        commit(std::integral_constant<int, 0>{}, 0);
+        __syncthreads();
+    }
+    if constexpr (NTT > 0) {
+        static_for<NTT>([&](auto tt) __attribute__((always_inline)) { iteration(std::integral_constant<int, decltype(tt)::value % 3>{}, decltype(tt)::value); });
+    } else {
+        for (int t = 0; t < NT; t += 3) {
+            iteration(std::integral_constant<int, 0>{}, t);
+            if (t + 1 < NT) iteration(std::integral_constant<int, 1>{}, t + 1);
+            if (t + 2 < NT) iteration(std::integral_constant<int, 2>{}, t + 2);
+        }
+    }
+    if (vh == 0) {   // the partial sums (one per group of rows) meet in LDS (the tiles are done with: the last barrier)
+        float* red = reinterpret_cast<float*>(smem);   // [NPG][D]
+        *reinterpret_cast<f32x8*>(red + pg * D + 8 * kc) = nacc;
+        __syncthreads();
+        if (tid < D) {
+            float sum = 0.f;
+#pragma unroll
+            for (int g = 0; g < NPG; g++) sum += red[g * D + tid];
+            a.Nst[((size_t)bh * a.NCS + cc) * D + tid] = sum;
+        }
+    }
+    };
+
+    auto multiply = [&]() __attribute__((always_inline)) {
+    SwzTransReader<T, D> krd;        // per-lane offsets of the transposing reads, computed once
+    krd.init(lane, (D / 128) * wave);
+    SwzTransReader<T, VW> vrd;
+    vrd.init(lane, 0);
+    f32x16 acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[mb][nb][x] = 0.f;
+    auto compute = [&](int t) __attribute__((always_inline)) {
         const T* kt = reinterpret_cast<const T*>(ks + (t % ST) * Cfg::K_BYTES);
         const T* vt = reinterpret_cast<const T*>(vs + (t % ST) * Cfg::V_BYTES);
         // the operand reads of a contraction step run one step ahead of its MFMAs (read, wait, multiply in turns left the
@@ -191,123 +317,19 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
 #pragma unroll
         for (int s = 0; s < NSTEP; s++) {
             if (s + 1 < NSTEP) rd(s + 1);
-            hook(s);
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) R::mma(acc[mb][nb], af[s & 1][mb], bf[s & 1][nb]);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (vh == 0) {   // the vector state's share of this tile
-            const char* kb = reinterpret_cast<const char*>(kt);
-#pragma unroll
-            for (int j = 0; j < PPT; j++) {
-                const int pos = PPT * pg + j;
-                float x[8];
-                unpack8<T>(*reinterpret_cast<const u32x4*>(kb + ZK::off(pos, 8 * kc)), x);
-                const float w2 = sw2[GRAN * t + pos];
-#pragma unroll
-                for (int e = 0; e < 8; e++) nacc[e] += x[e] * w2;
-            }
-        }
     };
-    // Iteration t (register set P = t % 3): the loads of tile t + 3 go out into the registers tile t left in the previous
-    // iteration; tile t is worked on, and between its MFMAs tile t + 1 moves to the LDS stage that tile t - 1 left behind the
-    // last barrier.  Two to three tiles are in flight while a tile is worked on.  The loads are ordinary ones, so that the compiler places the counted
-    // waits itself; it counts exactly in straight-line code (hence NTT: the default chunk's eight iterations are unrolled)
-    // and falls back to waiting for everything across a loop's back edge.  Loads issued by hand -- direct-to-LDS copies of
-    // K, or register loads from inline assembly -- gave wrong states now and then at full size as soon as a wait was a
-    // counted one: the compiler moves or stashes a register it believes written while the load is still in flight.  With
-    // one tile in flight and a wait for everything the kernel waited for memory latency in every iteration.
-    auto iteration = [&](auto set_tag, int t) __attribute__((always_inline)) {
-        constexpr int P = decltype(set_tag)::value, P1 = (P + 1) % 3;
-        if (t + 3 < NT) issue(std::integral_constant<int, P>{}, t + 3);
-        // (the vector work and LDS writes of the hand-over ride between the MFMAs: done in one piece before them they
-        // cost 1200 cycles per tile next to 1024 of MFMAs, measured)
-        compute(t, [&](int s) __attribute__((always_inline)) { if (t + 1 < NT) commit(std::integral_constant<int, P1>{}, t + 1, s); });
-        __syncthreads();
-    };
-
-    // The positions' weights.  Forward: w_j = exp(a_j - A_e) / sqrt(D) for both sums, e the chunk's last position.
-    // Reverse: rho_i = exp(A_e - A_i) / sqrt(D), e the last position BEFORE the chunk, times 1/n_i (matrix sum) or db_i
-    // (vector sum), the per-row scalars of the dQ pass.
-    const float log2scale = -0.5f * __log2f((float)D);
+    __syncthreads();   // (the weights are in LDS)
+    __syncthreads();   // (the first tile is)
     if constexpr (NTT > 0) {
-        // Their inputs are requested first and used behind the first tile's loads: the waits the compiler places for them
-        // then count the tile loads as "behind" and do not wait for those (requested after the tiles, the weights waited
-        // for all three tiles: 13 k cycles before the first iteration, measured).  The other two tiles' loads follow one
-        // by one, so that the first tile's data is not queued behind theirs.
-        constexpr int WPT = NTT * GRAN / 256;   // positions per thread
-        float x0[WPT], x1[WPT], x2[WPT];
-        double xg[WPT];
-        const float bend = a.beta2[poff + pe];
-        const double Gend = a.G2[goff + pe / GRAN];
-#pragma unroll
-        for (int n = 0; n < WPT; n++) {
-            int pos = p0 + tid + 256 * n;
-            pos = pos < S ? pos : S - 1;
-            xg[n] = a.G2[goff + pos / GRAN];
-            if (a.reverse) { x0[n] = a.beta2[poff + pos]; x1[n] = a.inv_n[poff + pos]; x2[n] = a.db[poff + pos]; }
-            else { x0[n] = a.alpha2[poff + pos]; x1[n] = 0.f; x2[n] = 0.f; }
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        issue(std::integral_constant<int, 0>{}, 0);
-#pragma unroll
-        for (int n = 0; n < WPT; n++) {
-            const int p = tid + 256 * n;
-            float w = 0.f, w2 = 0.f;
-            if (p0 + p < S) {
-                if (a.reverse) {
-                    const float rho = fast_exp2(bend - x0[n] + (float)(xg[n] - Gend) + log2scale);
-                    w = rho * x1[n];
-                    w2 = rho * x2[n];
-                } else {
-                    w = w2 = fast_exp2(x0[n] - bend + (float)(Gend - xg[n]) + log2scale);
-                }
-            }
-            sw[p] = w;
-            sw2[p] = w2;
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        issue(std::integral_constant<int, 1>{}, 1);   // (NT >= 2: a chunk is a multiple of 128 positions)
-        __syncthreads();   // the weights are in LDS
-        commit(std::integral_constant<int, 0>{}, 0, -1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
-        __syncthreads();
+        static_for<NTT>([&](auto tt) __attribute__((always_inline)) { compute(decltype(tt)::value); __syncthreads(); });
     } else {
-        issue(std::integral_constant<int, 0>{}, 0);
-        issue(std::integral_constant<int, 1>{}, 1);
-        if (2 < NT) issue(std::integral_constant<int, 2>{}, 2);
-        const float bend = a.beta2[poff + pe];
-        const double Gend = a.G2[goff + pe / GRAN];
-        for (int p = tid; p < L; p += 256) {
-            const int pos = p0 + p;
-            float w = 0.f, w2 = 0.f;
-            if (pos < S) {
-                if (a.reverse) {
-                    const float rho = fast_exp2(bend - a.beta2[poff + pos] + (float)(a.G2[goff + pos / GRAN] - Gend) + log2scale);
-                    w = rho * a.inv_n[poff + pos];
-                    w2 = rho * a.db[poff + pos];
-                } else {
-                    w = w2 = fast_exp2(a.alpha2[poff + pos] - bend + (float)(Gend - a.G2[goff + pos / GRAN]) + log2scale);
-                }
-            }
-            sw[p] = w;
-            sw2[p] = w2;
-        }
-        __syncthreads();   // the weights are in LDS
-        commit(std::integral_constant<int, 0>{}, 0, -1);
-        __syncthreads();
-    }
-    if constexpr (NTT > 0) {
-        static_for<NTT>([&](auto tt) __attribute__((always_inline)) { iteration(std::integral_constant<int, decltype(tt)::value % 3>{}, decltype(tt)::value); });
-    } else {
-        for (int t = 0; t < NT; t += 3) {
-            iteration(std::integral_constant<int, 0>{}, t);
-            if (t + 1 < NT) iteration(std::integral_constant<int, 1>{}, t + 1);
-            if (t + 2 < NT) iteration(std::integral_constant<int, 2>{}, t + 2);
-        }
+        for (int t = 0; t < NT; t++) { compute(t); __syncthreads(); }
     }
     // accumulator block (mb, nb): column (value) 32 nb + c32, rows (keys) 8 (r / 4) + 4 h + r % 4
     float* out = a.dC + ((size_t)bh * a.NCS + cc) * D * D + VW * vh;
@@ -320,17 +342,11 @@ __global__ __launch_bounds__(256) void chunk_sum_kernel(ChunkArgs a) {
                 const int k = (D / 4) * wave + 32 * mb + 8 * (r >> 2) + 4 * h + (r & 3);
                 out[(size_t)k * D + 32 * nb + c32] = acc[mb][nb][r];
             }
-    if (vh == 0) {   // the position groups' partial sums meet in LDS (the tiles are done with)
-        float* red = reinterpret_cast<float*>(smem);   // [NPG][D]
-        *reinterpret_cast<f32x8*>(red + pg * D + 8 * kc) = nacc;
-        __syncthreads();
-        if (tid < D) {
-            float sum = 0.f;
-#pragma unroll
-            for (int g = 0; g < NPG; g++) sum += red[g * D + tid];
-            a.Nst[((size_t)bh * a.NCS + cc) * D + tid] = sum;
-        }
-    }
+    if (vh == 0) __syncthreads();   // (the feeders' sum of the vector state)
+    };
+
+    if (feeder) feed();
+    else multiply();
 #endif
 }
 
@@ -445,10 +461,10 @@ static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     const size_t lds = Cfg::TILE_BYTES + 2 * (size_t)a.L * sizeof(float);
     if (a.L == 8 * GRAN) {   // the default chunk length
         if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 8>>(160 * 1024); e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 8>), grid, dim3(256), lds, st, a);
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 8>), grid, dim3(512), lds, st, a);
     } else {
         if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 0>>(160 * 1024); e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 0>), grid, dim3(256), lds, st, a);
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 0>), grid, dim3(512), lds, st, a);
     }
     // one carry kernel: the value-major one writes both layouts and the vector states
     if (a.CstT) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D>), dim3((D / 64) * (D / 64), a.BH), dim3(256), 0, st, a);
