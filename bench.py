@@ -240,17 +240,22 @@ def run_scan(ffi, steps, warmup, backward=False, shape=(1, 4, 2048, 1024), tag="
     h = torch.empty_like(q)
     ws, ws_n = ffi.workspace(ffi.OP_SCAN_FORWARD, B, NH, S, D, ffi.F32, dev)
     st, P = ffi.stream_ptr(), ffi.ptr
-    if backward:
+    if backward:   # a training step: the forward keeps its ungated output and normaliser sums for the backward
+        hu, bsum = torch.empty_like(q), torch.empty_like(f)
         dq, dk, dv, do = (torch.empty_like(q) for _ in range(4))
         df, di = torch.empty_like(f), torch.empty_like(i)
         wsb, wsb_n = ffi.workspace(ffi.OP_SCAN_BACKWARD, B, NH, S, D, ffi.F32, dev)
 
     def step():
-        ffi.check_rc(L.mlstm_scan_forward_ex(P(q), P(k), P(v), P(f), P(i), P(o), P(h), B, NH, S, D, ffi.F32, P(ws), ws_n, st),
-                     "mlstm_scan_forward_ex")
         if backward:
-            ffi.check_rc(L.mlstm_scan_backward_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(o), P(dq), P(dk), P(dv), P(df), P(di), P(do),
-                                                  B, NH, S, D, ffi.F32, P(wsb), wsb_n, st), "mlstm_scan_backward_ex")
+            ffi.check_rc(L.mlstm_scan_forward_save_ex(P(q), P(k), P(v), P(f), P(i), P(o), P(h), P(hu), P(bsum), B, NH, S, D, ffi.F32,
+                                                      P(ws), ws_n, st), "mlstm_scan_forward_save_ex")
+            ffi.check_rc(L.mlstm_scan_backward_saved_ex(P(dh), P(q), P(k), P(v), P(f), P(i), P(o), P(hu), P(bsum), P(dq), P(dk), P(dv),
+                                                        P(df), P(di), P(do), B, NH, S, D, ffi.F32, P(wsb), wsb_n, st),
+                         "mlstm_scan_backward_saved_ex")
+        else:
+            ffi.check_rc(L.mlstm_scan_forward_ex(P(q), P(k), P(v), P(f), P(i), P(o), P(h), B, NH, S, D, ffi.F32, P(ws), ws_n, st),
+                         "mlstm_scan_forward_ex")
 
     for _ in range(warmup):
         step()
@@ -270,12 +275,13 @@ def run_scan(ffi, steps, warmup, backward=False, shape=(1, 4, 2048, 1024), tag="
     kern = {name: ffi.timing_read(name) for name in names}
     ms_step = (t1 - t0) * 1e3 / steps
     BH = B * NH
-    # forward: q, k, v, o in, h out, f, i in (+ m); the backward adds dh in and six gradients out, and reads q, k, v, o, f, i again
-    bytes_compulsory = (5.0 * BH * S * D + 3.0 * BH * S) * 4 + (backward * (10.0 * BH * S * D + 4.0 * BH * S) * 4)
+    # forward: q, k, v, o in, h out, f, i in (+ m); the backward adds dh in and six gradients out, reads q, k, v, o, f, i again,
+    # and the ungated output travels from the one to the other
+    bytes_compulsory = (5.0 * BH * S * D + 3.0 * BH * S) * 4 + (backward * (12.0 * BH * S * D + 6.0 * BH * S) * 4)
     flops = BH * (S / 64.0) * (2 * 64 * D * D * 2 + 2 * 2 * D * 64 * 65 / 2 * 2)  # state update + read-out, in-chunk pairs
     st_ms = kern["scan_state"][0] / max(kern["scan_state"][1], 1)   # (average over the passes of a step)
     t_fl = flops / (st_ms * 1e-3) / 1e12 if st_ms else 0.0
-    flops *= 5 if backward else 1
+    flops *= 4 if backward else 1   # (the forward's walk and three more with other operands)
     return {
         "metric": "mLSTM scan-form %s, compulsory HBM GB/s, %s" % ("forward+backward" if backward else "forward", wl),
         "value": bytes_compulsory / (ms_step * 1e-3) / 1e9, "unit": "GB/s", "n_gpus": 1, "steps": steps,

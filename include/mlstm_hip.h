@@ -221,6 +221,17 @@ int mlstm_scan_forward_ex(const void* q, const void* k, const void* v, const voi
 int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
                            const void* o, void* dq, void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S,
                            int D, int dtype, void* workspace, size_t workspace_bytes, void* stream);
+/* The same pair for a training step that keeps what its backward would otherwise form again: the forward also leaves the
+ * ungated output h_ungated ([B,NH,S,D] fp32: numerator / n, before silu(o)) and the normaliser sums b ([B,NH,S]); the backward
+ * that is handed both skips its forward pass (one of its five walks over the sequence) and returns the same bits.  Null
+ * h_ungated and b make mlstm_scan_backward_saved_ex identical to mlstm_scan_backward_ex. */
+int mlstm_scan_forward_save_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
+                               void* h_ungated, float* b, int B, int NH, int S, int D, int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream);
+int mlstm_scan_backward_saved_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
+                                 const void* o, const void* h_ungated, const float* b, void* dq, void* dk, void* dv, void* df,
+                                 void* di, void* d_o, int B, int NH, int S, int D, int dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream);
 
 /*
  * sLSTM cell, forward and backward (fp32).  The reference lists the cell as an open item (README.md:9) and has no code

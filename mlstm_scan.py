@@ -6,4 +6,5 @@ mlstm_scan = _m.mlstm_scan
 # the backward of the scan form (the reference's kernel path has none) and the autograd function that carries it
 Scan_mLSTM = _m.Scan_mLSTM
 mlstm_scan_forward_hip = _m.mlstm_scan_forward_hip
+mlstm_scan_forward_save_hip = _m.mlstm_scan_forward_save_hip
 mlstm_scan_backward_hip = _m.mlstm_scan_backward_hip

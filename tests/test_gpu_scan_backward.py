@@ -78,6 +78,27 @@ def test_scan_backward_equals_gated_matmul_backward():
         assert_close(g, r, torch.float32, name)
 
 
+@pytest.mark.parametrize("S,D", [(100, 64), (192, 128), (700, 256), (300, 1024)])
+def test_kept_forward_gives_the_same_bits(S, D):
+    # the forward of a training step keeps its ungated output and normaliser sums; the backward that is handed them
+    # skips its own forward pass and must return what the recomputing backward returns, bit for bit
+    from mlstm_scan import mlstm_scan_backward_hip, mlstm_scan_forward_hip, mlstm_scan_forward_save_hip
+    q, k, v, f, i, dh, o = O.make_inputs(1, 3, S, D, torch.float32, seed=S + D, with_o=True)
+    dev = [x.cuda() for x in (dh, q, k, v, f, i, o)]
+    h, h_ungated, b = mlstm_scan_forward_save_hip(*dev[1:])
+    assert torch.equal(h, mlstm_scan_forward_hip(*dev[1:]))
+    hu_ref, _, b_ref = O.mlstm_forward_dense(q, k, v, f, i)      # (the scan form without its gate is the matmul form)
+    assert_close(h_ungated, hu_ref, torch.float32, "h_ungated")
+    assert_close(b, b_ref, torch.float32, "b")
+    kept = mlstm_scan_backward_hip(*dev, h_ungated, b)
+    plain = mlstm_scan_backward_hip(*dev)
+    for name, x, y in zip(NAMES, kept, plain):
+        assert torch.equal(x, y), name
+    check(kept, dh, q, k, v, f, i, o)
+    with pytest.raises(ValueError):
+        mlstm_scan_backward_hip(*dev, h_ungated, None)
+
+
 def test_scan_backward_is_repeatable():
     q, k, v, f, i, dh, o = (x.cuda() for x in O.make_inputs(1, 4, 300, 256, torch.float32, seed=25, with_o=True))
     a = run_backward(dh, q, k, v, f, i, o)

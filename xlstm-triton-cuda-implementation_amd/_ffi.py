@@ -84,6 +84,10 @@ def lib():
         L.mlstm_scan_forward_ex.argtypes = [vp] * 7 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_scan_backward_ex.restype = ci
         L.mlstm_scan_backward_ex.argtypes = [vp] * 13 + [ci] * 5 + [vp, sz, vp]
+        L.mlstm_scan_forward_save_ex.restype = ci
+        L.mlstm_scan_forward_save_ex.argtypes = [vp] * 8 + [fp] + [ci] * 5 + [vp, sz, vp]
+        L.mlstm_scan_backward_saved_ex.restype = ci
+        L.mlstm_scan_backward_saved_ex.argtypes = [vp] * 8 + [fp] + [vp] * 6 + [ci] * 5 + [vp, sz, vp]
         L.mlstm_timing_enable.restype = ci
         L.mlstm_timing_enable.argtypes = [ci]
         L.mlstm_timing_select.restype = ci
@@ -106,7 +110,7 @@ def lib():
 
 def exported_symbols():
     return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
-            "mlstm_scan_backward_ex", "slstm_saved_bytes", "slstm_workspace_bytes", "slstm_forward_ex", "slstm_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
+            "mlstm_scan_backward_ex", "mlstm_scan_forward_save_ex", "mlstm_scan_backward_saved_ex", "slstm_saved_bytes", "slstm_workspace_bytes", "slstm_forward_ex", "slstm_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",

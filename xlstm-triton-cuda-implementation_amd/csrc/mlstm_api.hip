@@ -255,7 +255,7 @@ int chunk_states_impl(const void* k, const void* v, const FwdWs& w, bool key_maj
 // matrix state walk, finish.  finish_mode as in ScanArgs; m_out / b_out (may be null) receive the stabiliser and the
 // normaliser sums.
 int scan_forward_impl(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h, float* m_out,
-                      float* b_out, const Sizes& z, int gate_dtype, int finish_mode, char* ws, hipStream_t st) {
+                      float* b_out, const Sizes& z, int gate_dtype, int finish_mode, char* ws, hipStream_t st, float* h_ungated = nullptr) {
     Carver c{ws, 0};
     double* G2 = c.take<double>(z.BH * z.NG);
     float* alpha2 = c.take<float>(z.BH * z.NG * 64);
@@ -281,7 +281,7 @@ int scan_forward_impl(const void* q, const void* k, const void* v, const void* f
     a.q = (const float*)q; a.k = (const float*)k; a.v = (const float*)v; a.o = (const float*)o; a.h = (float*)h;
     a.alpha2 = alpha2; a.beta2 = beta2; a.G2 = G2; a.M = m; a.P = P; a.Nst = Nst; a.hpart = hpart;
     a.BH = (int)z.BH; a.S = (int)z.S; a.D = (int)z.D; a.NC = (int)z.NG;
-    a.finish_mode = finish_mode; a.Bout = b_out; a.seg_state = seg_state;
+    a.finish_mode = finish_mode; a.Bout = b_out; a.Hun = h_ungated; a.seg_state = seg_state;
     return launch_scan(a, KS, st, scan_mark);
 }
 
@@ -730,11 +730,33 @@ int mlstm_scan_forward_ex(const void* q, const void* k, const void* v, const voi
     return scan_forward_impl(q, k, v, f, i, o, h, nullptr, nullptr, z, MLSTM_F32, 0, (char*)sc.p, st);
 }
 
+int mlstm_scan_forward_save_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
+                               void* h_ungated, float* b, int B, int NH, int S, int D, int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream) {
+    if (!q || !k || !v || !f || !i || !o || !h || !h_ungated || !b || B <= 0 || NH <= 0 || S <= 0) return MLSTM_EINVAL;
+    if (dtype != MLSTM_F32) return MLSTM_ESHAPE;
+    if (!(D == 64 || D == 128 || D == 256 || D == 512 || D == 1024) || S > 131072) return MLSTM_ESHAPE;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    const Sizes z = sizes_of(B, NH, S, D, MLSTM_F32);
+    Scratch sc;
+    if (int rc = sc.get(workspace, workspace_bytes, z.scan_fwd(), st)) return rc;
+    return scan_forward_impl(q, k, v, f, i, o, h, nullptr, b, z, MLSTM_F32, 0, (char*)sc.p, st, (float*)h_ungated);
+}
+
 int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
                            const void* o, void* dq, void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S, int D,
                            int dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return mlstm_scan_backward_saved_ex(dh_gated, q, k, v, f, i, o, nullptr, nullptr, dq, dk, dv, df, di, d_o, B, NH, S, D, dtype,
+                                        workspace, workspace_bytes, stream);
+}
+
+int mlstm_scan_backward_saved_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i,
+                                 const void* o, const void* h_ungated, const float* b, void* dq, void* dk, void* dv, void* df,
+                                 void* di, void* d_o, int B, int NH, int S, int D, int dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
     if (!dh_gated || !q || !k || !v || !f || !i || !o || !dq || !dk || !dv || !df || !di || !d_o || B <= 0 || NH <= 0 || S <= 0)
         return MLSTM_EINVAL;
+    if ((h_ungated == nullptr) != (b == nullptr)) return MLSTM_EINVAL;   // both kept, or neither
     if (dtype != MLSTM_F32) return MLSTM_ESHAPE;
     if (!(D == 64 || D == 128 || D == 256 || D == 512 || D == 1024) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -746,6 +768,7 @@ int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, c
     a.f = (const float*)f; a.i = (const float*)i; a.o = (const float*)o;
     a.dq = (float*)dq; a.dk = (float*)dk; a.dv = (float*)dv; a.df = (float*)df; a.di = (float*)di; a.d_o = (float*)d_o;
     a.BH = B * NH; a.S = S; a.D = D;
+    a.h_kept = (const float*)h_ungated; a.b_kept = b;
     return launch_scan_backward(a, (char*)sc.p, st, scan_mark);
 }
 

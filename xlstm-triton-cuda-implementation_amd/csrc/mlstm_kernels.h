@@ -192,6 +192,7 @@ struct ScanArgs {
     // reuses with other operands in the places of q, k and v.  Bout (may be null): the normaliser sums b_t, modes 0 and 1.
     int finish_mode;
     float* Bout;
+    float* Hun;           // mode 0 only, may be null: numerator / n next to the gated output (what a backward wants kept)
     // segments of the sequence that the state kernel runs side by side (filled in by launch_scan from scan_segments);
     // seg_state: scan_segment_state_bytes() bytes of scratch for the states at the segment ends, needed when nseg > 1
     float* seg_state;
@@ -212,6 +213,9 @@ struct ScanBwdArgs {
     const float* dhg; const float* q; const float* k; const float* v; const float* f; const float* i; const float* o;
     float* dq; float* dk; float* dv; float* df; float* di; float* d_o;
     int BH, S, D;
+    // the forward's ungated output and normaliser sums, if the caller kept them (both or neither): the forward is then not
+    // run again
+    const float* h_kept; const float* b_kept;
 };
 size_t scan_backward_workspace_bytes(int BH, int S, int D);
 int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*mark)(int, hipStream_t, bool));

@@ -418,7 +418,10 @@ __global__ __launch_bounds__(256) void scan_finish_kernel(ScanArgs a, int KS) {
             if (a.finish_mode == 0) {
                 const f32x4 ov = *reinterpret_cast<const f32x4*>(a.o + row * D + k);
 #pragma unroll
-                for (int e = 0; e < 4; e++) x[e] = x[e] * inv * (ov[e] / (1.0f + __expf(-ov[e])));
+                for (int e = 0; e < 4; e++) x[e] *= inv;
+                if (a.Hun) *reinterpret_cast<f32x4*>(a.Hun + row * D + k) = x;
+#pragma unroll
+                for (int e = 0; e < 4; e++) x[e] = x[e] * (ov[e] / (1.0f + __expf(-ov[e])));
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; e++) x[e] *= inv;

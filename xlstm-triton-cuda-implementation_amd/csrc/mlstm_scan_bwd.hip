@@ -276,7 +276,9 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
     const Plan p = plan_of(ws, BH, S, D);
     const size_t rows = (size_t)BH * S, N = rows * D;
     const int KS = scan_key_splits(BH, D), rb = row_blocks(rows);
-    float *h = p.T[0], *u = p.T[2], *yloc = p.T[3], *qr = p.T[4], *kr = p.T[5], *vr = p.T[6], *ur = p.T[7];
+    float *u = p.T[2], *yloc = p.T[3], *qr = p.T[4], *kr = p.T[5], *vr = p.T[6], *ur = p.T[7];
+    const float* h = a.h_kept ? a.h_kept : p.T[0];
+    const float* bsum = a.h_kept ? a.b_kept : p.b;
     float *RV = p.T[0], *RK = p.T[1];  // (h and dh are done with by then)
 
     mark(MLSTM_K_GATES, st, true);
@@ -290,10 +292,10 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
     auto fwd_gates = [&](ScanArgs& s) { s.alpha2 = p.alpha2; s.beta2 = p.beta2; s.G2 = p.G2; };
     auto rev_gates = [&](ScanArgs& s) { s.alpha2 = p.alpha2r; s.beta2 = p.beta2r; s.G2 = p.G2r; };
 
-    // the ungated forward output and its normaliser sums
-    {
+    // the ungated forward output and its normaliser sums, unless the caller kept them
+    if (!a.h_kept) {
         ScanArgs s = base; fwd_gates(s);
-        s.q = a.q; s.k = a.k; s.v = a.v; s.h = h; s.finish_mode = 1; s.Bout = p.b;
+        s.q = a.q; s.k = a.k; s.v = a.v; s.h = p.T[0]; s.finish_mode = 1; s.Bout = p.b;
         if (int rc = launch_scan(s, KS, st, mark)) return rc;
     }
     // the gradient of the ungated output: through the gate's backward, or, without a gate (o == null: the matmul
@@ -308,7 +310,7 @@ int launch_scan_backward(const ScanBwdArgs& a, char* ws, hipStream_t st, void (*
     }
 
     mark(MLSTM_K_SCAN_GLUE, st, true);
-    hipLaunchKernelGGL(scanbwd_rowstats_kernel, dim3(rb), dim3(256), 0, st, dh, h, p.b, p.m, u, p.db, p.db_rev, BH, S, D);
+    hipLaunchKernelGGL(scanbwd_rowstats_kernel, dim3(rb), dim3(256), 0, st, dh, h, bsum, p.m, u, p.db, p.db_rev, BH, S, D);
     hipLaunchKernelGGL(scanbwd_reverse_gates_kernel, dim3((unsigned)(((size_t)BH * NG * GRAN + 255) / 256)), dim3(256), 0, st, p.beta2, p.G2,
                        p.alpha2r, p.beta2r, p.G2r, BH, S, NG);
     hipLaunchKernelGGL(scanbwd_flip_kernel, dim3(rb), dim3(256), 0, st, a.q, qr, BH, S, D);

@@ -40,20 +40,43 @@ def mlstm_scan_forward_hip(q, k, v, f, i, o):
     return h
 
 
-def mlstm_scan_backward_hip(dh, q, k, v, f, i, o):
+def mlstm_scan_forward_save_hip(q, k, v, f, i, o):
+    """The forward of a training step: (h, h_ungated, b), the last two (the output before silu(o), the normaliser sums) kept
+    for ``mlstm_scan_backward_hip`` so that it does not form them again."""
+    B, NH, S, D = _check(q, k, v, f, i, o)
+    h, h_ungated = torch.empty_like(q), torch.empty_like(q)
+    b = torch.empty((B, NH, S), dtype=torch.float32, device=q.device)
+    ws, n = _ffi.workspace(_ffi.OP_SCAN_FORWARD, B, NH, S, D, _ffi.F32, q.device)
+    rc = _ffi.lib().mlstm_scan_forward_save_ex(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o),
+                                               _ffi.ptr(h), _ffi.ptr(h_ungated), _ffi.ptr(b), B, NH, S, D, _ffi.F32, _ffi.ptr(ws), n,
+                                               _ffi.stream_ptr())
+    _ffi.check_rc(rc, "mlstm_scan_forward_save_ex")
+    return h, h_ungated, b
+
+
+def mlstm_scan_backward_hip(dh, q, k, v, f, i, o, h_ungated=None, b=None):
     """Gradients (dq, dk, dv, df, di, do) of ``mlstm_scan`` for the output gradient ``dh``; df[..., 0] = 0 as in
-    mlstm_matmul.py:320-333.  The forward is recomputed inside: nothing but the inputs is needed."""
+    mlstm_matmul.py:320-333.  Nothing but the inputs is needed: the forward is run again inside, unless ``h_ungated`` and
+    ``b`` of ``mlstm_scan_forward_save_hip`` are handed over (the same bits either way)."""
     B, NH, S, D = _check(q, k, v, f, i, o)
     _ffi.require(dh, "dh", q.shape)
     if dh.dtype != torch.float32:
         raise TypeError("dh must be float32")
+    if (h_ungated is None) != (b is None):
+        raise ValueError("h_ungated and b go together")
+    if h_ungated is not None:
+        _ffi.require(h_ungated, "h_ungated", q.shape)
+        _ffi.require(b, "b", (B, NH, S))
+        if h_ungated.dtype != torch.float32 or b.dtype != torch.float32:
+            raise TypeError("h_ungated and b must be float32")
     dq, dk, dv, do = (torch.empty_like(q) for _ in range(4))
     df, di = torch.empty_like(f), torch.empty_like(i)
     ws, n = _ffi.workspace(_ffi.OP_SCAN_BACKWARD, B, NH, S, D, _ffi.F32, q.device)
-    rc = _ffi.lib().mlstm_scan_backward_ex(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o),
-                                           _ffi.ptr(dq), _ffi.ptr(dk), _ffi.ptr(dv), _ffi.ptr(df), _ffi.ptr(di), _ffi.ptr(do),
-                                           B, NH, S, D, _ffi.F32, _ffi.ptr(ws), n, _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_scan_backward_ex")
+    rc = _ffi.lib().mlstm_scan_backward_saved_ex(_ffi.ptr(dh), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i),
+                                                 _ffi.ptr(o), _ffi.ptr(h_ungated), _ffi.ptr(b), _ffi.ptr(dq), _ffi.ptr(dk),
+                                                 _ffi.ptr(dv), _ffi.ptr(df), _ffi.ptr(di), _ffi.ptr(do), B, NH, S, D, _ffi.F32,
+                                                 _ffi.ptr(ws), n, _ffi.stream_ptr())
+    _ffi.check_rc(rc, "mlstm_scan_backward_saved_ex")
     return dq, dk, dv, df, di, do
 
 
@@ -62,8 +85,9 @@ class Scan_mLSTM(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, f, i, o):
-        ctx.save_for_backward(q, k, v, f, i, o)
-        return mlstm_scan_forward_hip(q, k, v, f, i, o)
+        h, h_ungated, b = mlstm_scan_forward_save_hip(q, k, v, f, i, o)
+        ctx.save_for_backward(q, k, v, f, i, o, h_ungated, b)
+        return h
 
     @staticmethod
     def backward(ctx, dh):
