@@ -49,8 +49,19 @@ def test_benchmark_shape_twice():
     dev = gpu(wx, r, b)
     h, saved = slstm_forward_hip(*dev, forget_sigmoid=True)
     got = slstm_backward_hip(dh.cuda(), h, dev[1], saved, forget_sigmoid=True)
+    # the second run shares the memory system with a stream of large copies on another (default-priority) stream: the
+    # kernels' inputs arrive several steps ahead of their use, later or earlier than before, and nothing may change
+    side = torch.cuda.Stream()
+    big = torch.empty(64 * 1024 * 1024, device="cuda")
+    other = torch.empty_like(big)
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(40):
+            other.copy_(big)
     h2, saved2 = slstm_forward_hip(*dev, forget_sigmoid=True)
     got2 = slstm_backward_hip(dh.cuda(), h2, dev[1], saved2, forget_sigmoid=True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
     assert torch.equal(h, h2) and torch.equal(saved, saved2)
     for x, y in zip(got, got2):
         assert torch.equal(x, y)
