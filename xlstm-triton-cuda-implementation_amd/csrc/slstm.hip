@@ -10,9 +10,9 @@
 //   slstm_forward_kernel   four lanes per unit j, each with a quarter of row j of all four R_g: partial pre-activations from
 //                          h_{t-1} (LDS), summed over the four lanes; every lane then updates the cell of its unit.
 //                          Gate values and (c, n, m) are kept for the backward.
-//   slstm_backward_kernel  back through time, four lanes per unit k with quarters of column k of all four R_g: their sum is
-//                          what step t+1 sent back to h_t; every lane turns (dh_t + that, dc, dn) into the four
-//                          pre-activation gradients (= dWx_t).  The stabiliser m is a common scale of c and n that h
+//   slstm_backward_kernel  back through time: rows of 16 lanes form R^T delta_{t+1} for their four units (a sixteenth of the
+//                          gradient vector per lane, summed over the row), which is what step t+1 sent back to h_t; every
+//                          lane of a unit's quad turns (dh_t + that, dc, dn) into the four pre-activation gradients (= dWx_t).  The stabiliser m is a common scale of c and n that h
 //                          does not depend on, so it is held constant.
 //   slstm_dr_kernel        dR_g = sum_{b,t} dWx_t[g] h_{t-1}^T and db_g = sum_{b,t} dWx_t[g]: off the sequential path, in
 //                          slices of (b, t) whose partial sums a second kernel adds in a fixed order.
@@ -93,6 +93,12 @@ __device__ __forceinline__ float quad_sum(float x) {
     x += quad_perm<0xB1>(x);   // lanes 1, 0, 3, 2
     x += quad_perm<0x4E>(x);   // lanes 2, 3, 0, 1
     return x;
+}
+// Sum over the 16 lanes of a row (lanes 16a .. 16a+15), the same bits in all of them: rotations by 8 and 4, then the quad.
+__device__ __forceinline__ float row_sum(float x) {
+    x += quad_perm<0x128>(x);   // row_ror:8
+    x += quad_perm<0x124>(x);   // row_ror:4
+    return quad_sum(x);
 }
 // the value of lane q of a quad (three selects; is0..is2: q == 0, 1, 2)
 __device__ __forceinline__ float pick(bool is0, bool is1, bool is2, float a, float b, float c, float d) {
@@ -199,29 +205,33 @@ __global__ __launch_bounds__(4 * DH) void slstm_forward_kernel(const float* __re
     }
 }
 
-// Back through time with the same quads: lane q of unit k keeps, for all four gates, the quarter q of column k of R_g (what
-// unit k's output fed into the pre-activations of the units of that quarter), forms its quarter of R^T delta_{t+1} and
-// after the sum over the quad every lane has what step t + 1 sent back to h_t of its unit; all four lanes then form the four
-// pre-activation gradients alike, and lane q hands on and stores gradient q (delta in two buffers, taken in turns: one
-// barrier per step).  Lane q loads saved value q, and value 4 + q or, for q = 3, dh.
+// Back through time with the same quads, but what step t + 1 sends back to h_t -- R^T delta_{t+1}, a vector of 4 DH gradients
+// against DH outputs -- is formed by rows of 16 lanes: the four quads of a row own four units k, and lane p of the row takes
+// a sixteenth of the gradient vector for all four of them (DH / 4 gradients x 4 columns of R: DH registers, DH multiply-adds,
+// but only DH / 4 floats of LDS reads where a lane that served one unit alone read DH: the LDS pipeline was what the step
+// waited for).  The four sums meet over the row in four DPP exchanges; every lane keeps its own unit's, and all four lanes
+// of a quad then form the unit's four pre-activation gradients alike; lane q hands on and stores gradient q (delta in two
+// buffers, taken in turns: one barrier per step).  Lane q loads saved value q, and value 4 + q or, for q = 3, dh.
 template <int DH, bool FS>
 __global__ __launch_bounds__(4 * DH) void slstm_backward_kernel(const float* __restrict__ dh, const float* __restrict__ r,
                                                                 const float* __restrict__ saved, float* __restrict__ dwx, int NH,
                                                                 int S) {
-    constexpr int KQ = DH / 4;
-    constexpr int QS = 4 * KQ + 4;   // a quarter's units, and four floats so that the four quarters start in different banks
-    __shared__ __attribute__((aligned(16))) float delta[2][4 * QS];        // [buffer][quarter][unit * 4 + gate]
+    constexpr int PE = DH / 4;       // gradients per lane: a sixteenth of the 4 DH (in the order unit * 4 + gate)
+    constexpr int PS = PE + 4;       // ... and four floats, so that the 16 parts of a row's read start in different banks
+    __shared__ __attribute__((aligned(16))) float delta[2][16 * PS];       // [buffer][part][unit * 4 + gate within the part]
     __shared__ __attribute__((aligned(16))) float ring[PF][2][4 * DH];     // [slot][0: saved 0..3 | 1: saved 4..6, dh][unit * 4 + q]
     const int tid = threadIdx.x, k = tid >> 2, q = tid & 3, wave = tid >> 6;
     const bool is0 = q == 0, is1 = q == 1, is2 = q == 2;
     const int b = blockIdx.x / NH, hd = blockIdx.x % NH;
-    float rc[KQ][4];
+    const int part = tid & 15, k4 = (tid >> 4) * 4;   // the lane's part of the gradient vector; the first of its row's four units
+    float rc[PE][4];   // [gradient of the part][unit of the row]: R_g[j][k4 + u] for the part's (j, g)
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const float* src = r + (((size_t)hd * 4 + g) * DH + q * KQ) * DH + k;
-#pragma unroll
-        for (int jj = 0; jj < KQ; jj++) rc[jj][g] = src[(size_t)jj * DH];
+    for (int e = 0; e < PE; e++) {
+        const int f = part * PE + e, j = f >> 2, g = f & 3;
+        const f32x4 v = *reinterpret_cast<const f32x4*>(r + (((size_t)hd * 4 + g) * DH + j) * DH + k4);
+        rc[e][0] = v[0]; rc[e][1] = v[1]; rc[e][2] = v[2]; rc[e][3] = v[3];
     }
+    const int urow = k & 3;   // which of the row's units is this lane's own
     const size_t step_wx = (size_t)4 * NH * DH, step_h = (size_t)NH * DH, step_s = (size_t)7 * NH * DH;
     // (pointers that walk with the steps, from the last row down; f0, f1: the rows the ring takes next)
     const float* f0 = saved + ((size_t)b * S + S - 1) * step_s + ((size_t)q * NH + hd) * DH + k;
@@ -229,7 +239,7 @@ __global__ __launch_bounds__(4 * DH) void slstm_backward_kernel(const float* __r
                             : dh + ((size_t)b * S + S - 1) * step_h + (size_t)hd * DH + k;
     const size_t step1 = q < 3 ? step_s : step_h;
     float* dwp = dwx + ((size_t)b * S + S - 1) * step_wx + ((size_t)q * NH + hd) * DH + k;
-    const int mine_at = (k / KQ) * QS + (k % KQ) * 4 + q;   // where this lane's gradient goes in a delta buffer
+    const int mine_at = ((4 * k + q) / PE) * PS + (4 * k + q) % PE;   // where this lane's gradient goes in a delta buffer
     const unsigned ring_base = __builtin_amdgcn_readfirstlane(mlstm::lds_offset_of(&ring[0][0][0]) + wave * 256);
     auto fetch = [&](int u, bool more) __attribute__((always_inline)) {   // (before the start of the sequence: row 0 again)
         ring_load(f0, ring_base + (2 * u) * (4 * DH * 4));
@@ -239,22 +249,23 @@ __global__ __launch_bounds__(4 * DH) void slstm_backward_kernel(const float* __r
     constexpr int OPS = 3;   // per wave and step: the store of dwx, then two ring loads
 #pragma unroll
     for (int u = 0; u < PF; u++) fetch(u, S - 2 - u >= 0);
-    for (int e = tid; e < 4 * QS; e += 4 * DH) delta[0][e] = 0.f;   // (nothing comes back to the last step)
+    for (int e = tid; e < 16 * PS; e += 4 * DH) delta[0][e] = 0.f;   // (nothing comes back to the last step)
     float dc_next = 0.f, dn_next = 0.f;
     __syncthreads();
     // One step, the u-th of its round.  wait_n: how many of the wave's memory operations may still be under way when
     // the step takes its values from the ring.
     auto step = [&](int u, int t, int wait_n) __attribute__((always_inline)) {
-        const float* dcur = delta[u & 1] + q * QS;
-        f32x4 dl[KQ];
+        const float* dcur = delta[u & 1] + part * PS;
+        f32x4 dl[PE / 4];
 #pragma unroll
-        for (int jj = 0; jj < KQ; jj++) dl[jj] = *reinterpret_cast<const f32x4*>(dcur + jj * 4);
+        for (int e = 0; e < PE / 4; e++) dl[e] = *reinterpret_cast<const f32x4*>(dcur + 4 * e);
         float a[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int jj = 0; jj < KQ; jj++)
+        for (int e = 0; e < PE; e++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) a[g] += rc[jj][g] * dl[jj][g];
-        const float dhrec = quad_sum((a[0] + a[1]) + (a[2] + a[3]));
+            for (int x = 0; x < 4; x++) a[x] += rc[e][x] * dl[e >> 2][e & 3];
+        const float r0 = row_sum(a[0]), r1 = row_sum(a[1]), r2 = row_sum(a[2]), r3 = row_sum(a[3]);
+        const float dhrec = urow == 0 ? r0 : urow == 1 ? r1 : urow == 2 ? r2 : r3;
         ring_wait(wait_n);
         const int un = (u + 1) % PF;
         const f32x4 s0 = *reinterpret_cast<const f32x4*>(&ring[u][0][4 * k]);    // i~, log f, z, o
