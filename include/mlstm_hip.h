@@ -47,6 +47,10 @@ extern "C" {
  * cutlass-src-hopper/mlstm_forward.cu:201 suggests fusing away).  One layout for q, k, v and their gradients, one for
  * h and its gradient, one (without d) for the gates f, i and their gradients.  Rows must start on 16-byte boundaries:
  * base pointers 16-byte aligned, qkv / out strides multiples of 8 elements (16-bit types) or 4 (fp32).
+ * A layout in which the library WRITES (out for the forward's h; qkv and gates for the backward's gradients) must not
+ * overlap itself: an expanded view (a stride of 0 over more than one index) or interleaved rows would have several
+ * workgroups write one address, so such a layout is refused with MLSTM_EINVAL (pass a dense copy instead).  Tensors that
+ * are only read may overlap.
  * gate_form says what `f` holds: the forget gate's pre-activation (the reference's input, mlstm_matmul.py:57), its
  * log-sigmoid, or the cumulative sum of the log-sigmoid over the positions of each head (what mlstm_matmul.py:57-58
  * compute first; fp32 gates only: the sum reaches 1e3..1e4 and 16-bit types cannot hold it).  The backward returns
@@ -120,6 +124,9 @@ int mlstm_forward_ex(const void* q, const void* k, const void* v, const void* f,
  * that size are rejected with MLSTM_EWORKSPACE.  All calls on one GPU share the one array: two calls that overlap in
  * time on the same GPU (different streams or threads) race; calls on one stream are ordered and safe.
  * (With mlstm_timing_enable on, events are created around the launches; leave it off in such callers.)
+ * The first call on a device looks up the array's address (a mutex and a runtime query) and the first launch of each
+ * kernel variant raises that kernel's LDS limit (hipFuncSetAttribute): neither belongs inside a stream capture.  Make
+ * one ordinary call per device and shape class before capturing (mlstm_init() does the address lookup alone).
  */
 #define MLSTM_NOALLOC_MAX_WORKSPACE (8u << 20)
 int mlstm_forward_noalloc_ex(const void* q, const void* k, const void* v, const void* f, const void* i, void* h, float* m,
@@ -308,13 +315,18 @@ int mlstm_chunk_length_for(int S, int D, int dtype);
  * Fail-safe of the eight-wave row kernel, no counterpart in the reference.  Inside a workgroup its producer waves wait
  * for an LDS counter before they reuse a buffer; the wait is bounded, and if it ever expires (a bug: it cannot in a
  * correct build) the kernel sets a per-GPU error word and runs on to its end instead of hanging the GPU.
- * mlstm_kernel_error waits for the current device's work, returns MLSTM_EKERNEL if the word is set (results since the
- * last call are then not to be trusted) and clears it, 0 otherwise.  mlstm_set_spin_limit is the test aid for it:
+ * mlstm_kernel_error waits for ALL work of the current device (hipDeviceSynchronize: every stream, the non-blocking
+ * ones included), returns MLSTM_EKERNEL if the word is set (results since the last call are then not to be trusted) and
+ * clears it, 0 otherwise.  Work launched by other threads between its read and its clear can lose an error.  mlstm_set_spin_limit is the test aid for it:
  * limit > 0 replaces the bound (loop iterations), limit < 0 makes every such wait count as expired without waiting
  * (the results of that run are undefined), 0 restores the default.  Process-wide.
  */
 int mlstm_kernel_error(void);
 int mlstm_set_spin_limit(int limit);
+
+/* Per-device set-up that the first call on a device would otherwise do (the addresses of the library's static device
+ * arrays): call with that device current; returns 0 or a HIP error.  Optional, and idempotent. */
+int mlstm_init(void);
 
 /* Library version string, e.g. "mlstm_hip 0.1 gfx950". */
 const char* mlstm_version(void);

@@ -44,6 +44,30 @@ def test_noalloc_forward_matches_forward_ex_on_two_calls_in_a_row():
         assert torch.equal(h0, h1) and torch.equal(m0, m1) and torch.equal(b0, b1), (S, D, dtype)
 
 
+def test_noalloc_forward_leaves_device_memory_as_it_found_it():
+    """After one warm-up call per shape (which loads the kernels and looks up the scratch array), further calls must not
+    change the device's free memory: nothing is allocated or freed, stream-ordered or otherwise."""
+    B, NH, S, D = 1, 2, 1536, 128
+    q, k, v, f, i, _ = [x.cuda() for x in O.make_inputs(B, NH, S, D, torch.bfloat16, seed=5, f_mean=2.0)]
+    h = torch.empty_like(q)
+    m = torch.empty((B, NH, S), device="cuda", dtype=torch.float32)
+    b = torch.empty_like(m)
+    L = ffi.lib()
+    assert L.mlstm_init() == 0
+    args = (ffi.ptr(q), ffi.ptr(k), ffi.ptr(v), ffi.ptr(f), ffi.ptr(i), ffi.ptr(h), ffi.ptr(m), ffi.ptr(b), B, NH, S, D, ffi.BF16, ffi.BF16,
+            ffi.stream_ptr())
+    ffi.check_rc(L.mlstm_forward_noalloc_ex(*args), "warm-up")
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        ffi.check_rc(L.mlstm_forward_noalloc_ex(*args), "mlstm_forward_noalloc_ex")
+        free_during, _ = torch.cuda.mem_get_info()
+        assert free_during == free0
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0
+
+
 def test_noalloc_forward_rejects_shapes_beyond_its_scratch():
     B, NH, S, D = 4, 8, 4096, 256
     L = ffi.lib()

@@ -98,6 +98,8 @@ def lib():
         L.mlstm_chunk_length_for.argtypes = [ci] * 3
         L.mlstm_kernel_error.restype = ci
         L.mlstm_kernel_error.argtypes = []
+        L.mlstm_init.restype = ci
+        L.mlstm_init.argtypes = []
         L.mlstm_set_spin_limit.restype = ci
         L.mlstm_set_spin_limit.argtypes = [ci]
         L.mlstm_force_generic_kernels.restype = ci
@@ -114,7 +116,7 @@ def exported_symbols():
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
-            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit"]
+            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init"]
 
 
 KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
@@ -182,6 +184,27 @@ def require_rows(t, name, shape=None, like=None):
         raise ValueError(f"{name}: the head dimension must be contiguous (strides {t.stride()})")
     if like is not None and tuple(t.stride()) != tuple(like.stride()):
         raise ValueError(f"{name} must have the layout of its companion (strides {t.stride()} against {like.stride()})")
+
+
+def overlaps(t):
+    """Does the view address one element more than once (an expanded tensor, stride 0, or any other self-overlap)?
+    Sufficient test, the one the library applies to tensors it writes: in the order of their strides every dimension
+    must step over everything the smaller ones span."""
+    extent = 1
+    for n, s in sorted(((n, s) for n, s in zip(t.shape, t.stride()) if n > 1), key=lambda p: p[1]):
+        if s < extent:
+            return True
+        extent += (n - 1) * s
+    return False
+
+
+def dense_unless_disjoint(*ts):
+    """The tensors as they are, or, if any of them overlaps itself, contiguous copies of all of them.  Gradients are
+    laid out like their tensors: for an expanded input (``f.expand(...)`` to share gates over heads) that layout would
+    make several workgroups write one address.  With a dense copy autograd's own backward of the expansion does the sum."""
+    if any(overlaps(t) for t in ts):
+        return tuple(t.contiguous() for t in ts)
+    return ts
 
 
 def dense_in_order_of(t):

@@ -1,6 +1,7 @@
 // C ABI of libmlstm_hip.so: argument checks, workspace carving and the launch sequences.
 #include <hip/hip_runtime.h>
 #include <mutex>
+#include <utility>
 #include <vector>
 #include "mlstm_kernels.h"
 
@@ -135,9 +136,29 @@ Sizes sizes_of(int B, int NH, int S, int D, int dtype_arg) {
 }
 bool good_shape(int D, int dtype) { return D == 64 || D == 128 || D == 256 || (dtype == MLSTM_F32 && (D == 512 || D == 1024)); }
 
+// Do the elements of a [B,NH,S] grid of rows of `row` elements each stay apart under these strides?  (Sufficient test:
+// taken in the order of their strides, every dimension must step over everything the smaller ones span.)  A tensor the
+// library WRITES must pass it: with an expanded view (a zero stride) or any other overlap several workgroups would
+// write one address and the last writer would win.
+bool non_overlapping(long long B, long long NH, long long S, long long sb, long long sh, long long ss, long long row) {
+    long long n[3] = {B, NH, S}, st[3] = {sb, sh, ss};
+    for (int a = 0; a < 3; a++)
+        for (int b = a + 1; b < 3; b++)
+            if (st[b] < st[a]) { std::swap(st[a], st[b]); std::swap(n[a], n[b]); }
+    long long extent = row;
+    for (int a = 0; a < 3; a++) {
+        if (n[a] <= 1) continue;
+        if (st[a] < extent) return false;
+        extent += (n[a] - 1) * st[a];
+    }
+    return true;
+}
+
 // The caller's layout into z (null: everything dense).  Rows of q, k, v, h must start on 16-byte boundaries, and the
-// tile copies address a tile's 64 rows with 32-bit byte offsets.
-int apply_layout(Sizes& z, const mlstm_layout* L, int NH, int gate_dtype, std::initializer_list<const void*> row_tensors) {
+// tile copies address a tile's 64 rows with 32-bit byte offsets.  written_qkv / written_out / written_gates: the call
+// writes tensors in that layout (gradients, h), which must then not overlap themselves.
+int apply_layout(Sizes& z, const mlstm_layout* L, int NH, int gate_dtype, std::initializer_list<const void*> row_tensors, bool written_qkv,
+                 bool written_out, bool written_gates) {
     if (!L) return 0;
     const long long el = (long long)z.el;
     auto good = [&](long long b, long long h, long long s) {
@@ -147,6 +168,10 @@ int apply_layout(Sizes& z, const mlstm_layout* L, int NH, int gate_dtype, std::i
     if (L->gate_stride_b < 0 || L->gate_stride_h < 0 || L->gate_stride_s < 1) return MLSTM_EINVAL;
     if (L->gate_form != MLSTM_GATE_RAW && L->gate_form != MLSTM_GATE_LOGSIGMOID && L->gate_form != MLSTM_GATE_CUMSUM) return MLSTM_EINVAL;
     if (L->gate_form == MLSTM_GATE_CUMSUM && gate_dtype != MLSTM_F32) return MLSTM_EINVAL;
+    const long long B = (long long)z.BH / NH, S = (long long)z.S, D = (long long)z.D;
+    if (written_qkv && !non_overlapping(B, NH, S, L->qkv_stride_b, L->qkv_stride_h, L->qkv_stride_s, D)) return MLSTM_EINVAL;
+    if (written_out && !non_overlapping(B, NH, S, L->out_stride_b, L->out_stride_h, L->out_stride_s, D)) return MLSTM_EINVAL;
+    if (written_gates && !non_overlapping(B, NH, S, L->gate_stride_b, L->gate_stride_h, L->gate_stride_s, 1)) return MLSTM_EINVAL;
     for (const void* p : row_tensors)
         if (p && (reinterpret_cast<size_t>(p) & 15)) return MLSTM_EINVAL;
     z.la = Lay{L->qkv_stride_b, L->qkv_stride_h, L->qkv_stride_s, NH};
@@ -355,11 +380,17 @@ int mlstm_set_spin_limit(int limit) {
     return 0;
 }
 
+int mlstm_init(void) { return symbols_of_current_device(nullptr, nullptr); }
+
 int mlstm_kernel_error(void) {
     int* word = nullptr;
     if (int rc = symbols_of_current_device(nullptr, &word)) return rc;
+    // Every stream of the device, the non-blocking ones included (a plain copy on the null stream waits for the
+    // blocking streams only); with the device idle the read and the clear below cannot lose an error in between.
+    hipError_t e = hipDeviceSynchronize();
+    if (e != hipSuccess) return (int)e;
     int value = 0;
-    hipError_t e = hipMemcpy(&value, word, sizeof(int), hipMemcpyDeviceToHost);   // (waits for the device's work)
+    e = hipMemcpy(&value, word, sizeof(int), hipMemcpyDeviceToHost);
     if (e != hipSuccess) return (int)e;
     if (value != 0) {
         const int zero = 0;
@@ -435,7 +466,7 @@ int mlstm_forward_lx(const void* q, const void* k, const void* v, const void* f,
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h})) return rc;
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h}, false, true, false)) return rc;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -481,7 +512,7 @@ int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const voi
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h})) return rc;
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, h}, false, true, false)) return rc;
     if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
@@ -643,7 +674,7 @@ int mlstm_backward_lx(const void* dh, const void* q, const void* k, const void* 
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv})) return rc;
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv}, true, false, true)) return rc;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;
     return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, z, D, dtype, gate_dtype, (char*)sc.p, st);
@@ -669,7 +700,7 @@ int mlstm_backward_saved_lx(const void* dh, const void* q, const void* k, const 
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     Sizes z = sizes_of(B, NH, S, D, dtype_arg);
-    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv})) return rc;
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh, q, k, v, h, dq, dk, dv}, true, false, true)) return rc;
     if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd(), st)) return rc;

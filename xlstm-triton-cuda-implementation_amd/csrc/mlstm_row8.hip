@@ -267,6 +267,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             }
         };
         // hand the fragments of tile j to the consumers of the same rows; they have copied tile j-1's long ago
+        bool expired = false;
         auto publish = [&](const f32x16& s0, const f32x16& s1, int j) {
             frag f00 = R::from_acc(s0, 0), f01 = R::from_acc(s0, 1), f10 = R::from_acc(s1, 0), f11 = R::from_acc(s1, 1);
             if (j > 0) {
@@ -275,11 +276,12 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 volatile unsigned* c = pcnt + rg;
                 if (a.spin_limit < 0) {   // test aid: every wait counts as expired, without waiting
                     if (lane == 0 && j == 1) atomicOr(a.err, 1);
-                } else {
-                    int spins = 0;
+                } else if (!expired) {    // (once a wait has expired in this wave the later ones are not waited for either:
+                    int spins = 0;        //  the results are lost anyway, and the kernel should end soon)
                     while (*c < 2u * (unsigned)j) {
                         if (spins++ >= a.spin_limit) {
                             if (lane == 0) atomicOr(a.err, 1);
+                            expired = true;
                             break;
                         }
                         __builtin_amdgcn_s_sleep(1);

@@ -49,6 +49,8 @@ def mlstm_forward_hip(q, k, v, f, i, precise=False, gate_form="raw"):
     """Returns (h, m, b): h [B,NH,S,D] in q's dtype and dimension order in memory, m and b [B,NH,S] fp32 (reference
     mlstm_matmul.py:373-378).  gate_form: what f holds ("raw" pre-activations as in the reference, "logsigmoid", or
     "cumsum" of the log-sigmoid over the positions; fp32 gates only for the last)."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     h = _ffi.dense_in_order_of(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
@@ -65,6 +67,8 @@ def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False,
     """Returns (dq, dk, dv, df, di) (reference mlstm_matmul.py:384-405), each in the layout of the tensor it is the
     gradient of; df is the gradient of whatever f held (gate_form).  h, m, b: the forward's outputs, or None to have
     them recomputed."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     if not dh.is_cuda or tuple(dh.shape) != tuple(q.shape):
         raise ValueError(f"dh must be a GPU tensor of q's shape, got {tuple(dh.shape)} on {dh.device}")
@@ -93,6 +97,8 @@ def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False,
 def mlstm_forward_save_hip(q, k, v, f, i, precise=False, gate_form="raw"):
     """Forward of a training step.  Returns (h, m, b, saved): as mlstm_forward_hip, plus what the backward can reuse (the
     states at the chunk ends of a long 16-bit sequence; None for shapes that do not run in chunks)."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     h = _ffi.dense_in_order_of(q)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
@@ -110,6 +116,8 @@ def mlstm_forward_save_hip(q, k, v, f, i, precise=False, gate_form="raw"):
 
 def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=False, gate_form="raw"):
     """Backward of a training step with the forward's outputs and its saved states (mlstm_forward_save_hip)."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
     if not dh.is_cuda or tuple(dh.shape) != tuple(q.shape):
         raise ValueError(f"dh must be a GPU tensor of q's shape, got {tuple(dh.shape)} on {dh.device}")
