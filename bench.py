@@ -116,17 +116,21 @@ def cpu_baseline_torch(host, S, D, heads=2):
             "tokens_per_s": heads * S / dt}
 
 
-def chunk_work(S, D, BH, chunk, el):
-    """Flops the kernels execute per step in chunks of `chunk`, and the column kernel's share, with its compulsory bytes."""
+def chunk_work(S, D, BH, chunk, el, precise=False):
+    """Flops the kernels execute per step in chunks of `chunk`, and the column kernel's share, with its compulsory bytes.
+    ``precise``: split mode, every second product of a pair and every product with a state or a weighted row runs twice (on
+    the hi and on the lo term), and the states are twice the bytes."""
     lens = [min(chunk, S - c0) for c0 in range(0, S, chunk)]
     pair_unit = float(D) * sum(n * (n + 1) for n in lens) * BH            # one product over the (query, key) pairs inside chunks
     state_rows = float(sum(lens[1:])) * BH                                 # positions that read a forward state
     state_keys = float(sum(lens[:-1])) * BH                                # positions that read a reverse state
     sums = 2.0 * D * D * (sum(lens[:-1]) + sum(lens[1:])) * BH             # chunk sums, both directions (2 D^2 per position)
-    executed = 8.0 * pair_unit + 2.0 * D * D * 2 * state_rows + 2.0 * D * D * 2 * state_keys + sums
-    col_flops = 4.0 * pair_unit + 2.0 * D * D * 2 * state_keys            # four products per pair, two with the reverse state
+    two = 2.0 if precise else 1.0
+    executed = (12.0 if precise else 8.0) * pair_unit + two * (2.0 * D * D * 2 * state_rows + 2.0 * D * D * 2 * state_keys + sums)
+    # four products per pair (six in split mode), two with the reverse state
+    col_flops = (6.0 if precise else 4.0) * pair_unit + two * 2.0 * D * D * 2 * state_keys
     tiles_met = sum((n // 64 + 1) / 2.0 * n for n in lens)
-    col_bytes = BH * (S * D * el * 6 + tiles_met * 4 + (len(lens) - 1) * (D * D * el + 4.0 * D))
+    col_bytes = BH * (S * D * el * 6 + tiles_met * 4 + (len(lens) - 1) * (two * D * D * el + 4.0 * D))
     return executed, col_flops, col_bytes
 
 
@@ -190,7 +194,7 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
     chunk = int(L.mlstm_chunk_length_for(S, D, dt_code))
     el = torch.empty(0, dtype=dtype).element_size()
     if chunk > 0 and (S + 63) // 64 <= 1024:
-        executed, col_flops, col_bytes = chunk_work(S, D, BH, chunk, el)
+        executed, col_flops, col_bytes = chunk_work(S, D, BH, chunk, el, precise)
     else:
         # every key tile: 8 products executed (dH V^T in both backward kernels), 4 of them in the column kernel; the split
         # mode runs each of the 4 second products (P V, G K, G^T Q, W^T dH) a second time on the low-order terms

@@ -33,8 +33,9 @@ extern "C" {
  * size.  With MLSTM_PRECISE every such operand enters its product as two terms, hi + lo, each in the element type
  * (two MFMAs per fragment), and the forward hands the low-order part of h to the backward (the `saved` buffer of
  * mlstm_forward_save_ex, or a recomputation), which makes the results agree with an fp32 evaluation of the
- * reference's formulas (mlstm_matmul.py:104-118, :336-365) to rtol 2e-2 / atol 2e-3 element by element.  Price:
- * the generic kernels without chunking, and half as many MFMAs again.
+ * reference's formulas (mlstm_matmul.py:104-118, :336-365) to rtol 2e-2 / atol 2e-3 element by element.  Long
+ * sequences run in chunks in this mode too, with every chunk state kept as two terms.  Price: the four-wave kernels
+ * instead of the eight-wave ones, and half as many MFMAs again.
  */
 #define MLSTM_PRECISE 0x100
 
@@ -71,6 +72,7 @@ typedef struct mlstm_layout {
 #define MLSTM_ESHAPE (-2)      /* head dimension / sequence length not supported by this build */
 #define MLSTM_EWORKSPACE (-3)  /* caller workspace smaller than mlstm_workspace_bytes() */
 #define MLSTM_EKERNEL (-4)     /* a kernel's bounded wait expired (mlstm_kernel_error) */
+#define MLSTM_ESAVED (-5)      /* a backward was given a `saved` buffer written for another shape or setting (mlstm_kernel_error) */
 
 /* operations, for mlstm_workspace_bytes */
 #define MLSTM_OP_FORWARD 0
@@ -149,8 +151,11 @@ int mlstm_backward_ex(const void* dh, const void* q, const void* k, const void* 
  * chunks, the states at the chunk ends and the gate pre-pass, so that the backward does not form them again.  `saved` is caller-owned device
  * memory of mlstm_saved_state_bytes(...) bytes (0 for shapes that do not run in chunks: saved may then be NULL), written
  * by mlstm_forward_save_ex and read by mlstm_backward_saved_ex for the same inputs and the same dtype argument; the
- * chunk length (mlstm_set_chunk_length) must not change in between (saved_bytes must equal mlstm_saved_state_bytes
- * at the time of either call, which catches a change of the number of chunks).  Otherwise as mlstm_forward_ex / mlstm_backward_ex, with h, m
+ * process-wide settings (mlstm_set_chunk_length, mlstm_force_generic_kernels) must not change in between.  saved_bytes
+ * must equal mlstm_saved_state_bytes at the time of either call (checked on the host), and the buffer starts with a
+ * header -- shape, dtype argument, chunk length, kernel switch -- that the forward writes and the backward compares ON
+ * THE DEVICE, without a host round trip: a mismatch sets the per-GPU error word, the backward's results are then
+ * garbage (all reads stay inside the buffers), and mlstm_kernel_error() reports MLSTM_ESAVED.  Otherwise as mlstm_forward_ex / mlstm_backward_ex, with h, m
  * and b required in the backward.  MLSTM_EWORKSPACE also reports a `saved` buffer that is missing or too small.
  */
 size_t mlstm_saved_state_bytes(int B, int NH, int S, int D, int dtype);
@@ -316,7 +321,8 @@ int mlstm_chunk_length_for(int S, int D, int dtype);
  * for an LDS counter before they reuse a buffer; the wait is bounded, and if it ever expires (a bug: it cannot in a
  * correct build) the kernel sets a per-GPU error word and runs on to its end instead of hanging the GPU.
  * mlstm_kernel_error waits for ALL work of the current device (hipDeviceSynchronize: every stream, the non-blocking
- * ones included), returns MLSTM_EKERNEL if the word is set (results since the last call are then not to be trusted) and
+ * ones included), returns MLSTM_EKERNEL if an expired wait set the word (MLSTM_ESAVED if only a mismatched `saved`
+ * buffer did, see mlstm_forward_save_ex) (results since the last call are then not to be trusted) and
  * clears it, 0 otherwise.  Work launched by other threads between its read and its clear can lose an error.  mlstm_set_spin_limit is the test aid for it:
  * limit > 0 replaces the bound (loop iterations), limit < 0 makes every such wait count as expired without waiting
  * (the results of that run are undefined), 0 restores the default.  Process-wide.

@@ -161,3 +161,54 @@ def test_layouts_the_kernels_cannot_take_are_rejected():
         mlstm_forward_hip(q, k, v, f, i, gate_form="cumsum")
     with pytest.raises(ValueError):
         mlstm_forward_hip(q, k, v, f, i, gate_form="sigmoid")
+
+
+def test_expanded_inputs_get_the_summed_gradient():
+    """Gates shared over the heads (f.expand) and a query shared over the batch (q.expand): the gradient with respect to
+    the unexpanded tensor is the sum over the copies, as with dense inputs; gradient buffers never alias."""
+    from mlstm_matmul import Triton_mLSTM
+    B, NH, S, D = 2, 3, 200, 64
+    q, k, v, f, i, dh = (x.cuda() for x in O.make_inputs(B, NH, S, D, torch.float32, seed=41))
+    f1, i1, q1 = f[:, :1].clone().requires_grad_(True), i[:, :1].clone().requires_grad_(True), q[:1].clone().requires_grad_(True)
+    k1, v1 = k.clone().requires_grad_(True), v.clone().requires_grad_(True)
+    Triton_mLSTM.apply(q1.expand(B, NH, S, D), k1, v1, f1.expand(B, NH, S), i1.expand(B, NH, S)).backward(dh)
+    dense = [q1.detach().expand(B, NH, S, D).contiguous().requires_grad_(True), k.clone().requires_grad_(True), v.clone().requires_grad_(True),
+             f1.detach().expand(B, NH, S).contiguous().requires_grad_(True), i1.detach().expand(B, NH, S).contiguous().requires_grad_(True)]
+    Triton_mLSTM.apply(*dense).backward(dh)
+    assert_close(q1.grad, dense[0].grad.sum(0, keepdim=True), torch.float32, "dq of the shared query")
+    assert_close(f1.grad, dense[3].grad.sum(1, keepdim=True), torch.float32, "df of the shared gates")
+    assert_close(i1.grad, dense[4].grad.sum(1, keepdim=True), torch.float32, "di of the shared gates")
+    assert torch.equal(k1.grad, dense[1].grad) and torch.equal(v1.grad, dense[2].grad)
+
+
+def test_library_refuses_overlapping_layouts_for_tensors_it_writes():
+    from _mlstm_pkg import submodule
+    ffi = submodule("_ffi")
+    B, NH, S, D = 2, 2, 128, 64
+    q, k, v, f, i, dh = (x.cuda() for x in O.make_inputs(B, NH, S, D, torch.float32, seed=42))
+    h = torch.empty_like(q)
+    g = [torch.empty_like(q) for _ in range(3)] + [torch.empty_like(f) for _ in range(2)]
+    L = ffi.lib()
+    ws, n = ffi.workspace(ffi.OP_BACKWARD, B, NH, S, D, ffi.F32, q.device)
+
+    def backward(lay):
+        return L.mlstm_backward_lx(ffi.ptr(dh), ffi.ptr(q), ffi.ptr(k), ffi.ptr(v), ffi.ptr(f), ffi.ptr(i), None, None, None, *[ffi.ptr(x) for x in g],
+                                   B, NH, S, D, ffi.F32, ffi.F32, lay, ffi.ptr(ws), n, ffi.stream_ptr())
+
+    good = ffi.layout(q, h, f)
+    assert backward(good) == 0
+    shared_gates = ffi.Layout(*[getattr(good, n_) for n_, _ in ffi.Layout._fields_])
+    shared_gates.gate_h = 0                       # gates shared over the heads: df, di would alias
+    assert backward(shared_gates) == -1
+    shared_q = ffi.Layout(*[getattr(good, n_) for n_, _ in ffi.Layout._fields_])
+    shared_q.qkv_b = 0                            # q, k, v shared over the batch: dq, dk, dv would alias
+    assert backward(shared_q) == -1
+    # the forward only reads q, k, v and the gates: the same layouts are fine there, an overlapping h is not
+    ws2, n2 = ffi.workspace(ffi.OP_FORWARD, B, NH, S, D, ffi.F32, q.device)
+    fwd = lambda lay: L.mlstm_forward_lx(ffi.ptr(q), ffi.ptr(k), ffi.ptr(v), ffi.ptr(f), ffi.ptr(i), ffi.ptr(h), None, None, B, NH, S, D,
+                                         ffi.F32, ffi.F32, lay, ffi.ptr(ws2), n2, ffi.stream_ptr())
+    assert fwd(shared_gates) == 0 and fwd(shared_q) == 0
+    shared_h = ffi.Layout(*[getattr(good, n_) for n_, _ in ffi.Layout._fields_])
+    shared_h.out_h = 0
+    assert fwd(shared_h) == -1
+    torch.cuda.synchronize()

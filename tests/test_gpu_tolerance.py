@@ -19,16 +19,22 @@ from tests.helpers import GRAD_NAMES, assert_close, assert_matches_oracle, liter
 pytestmark = pytest.mark.gpu
 
 mm = submodule("mlstm_matmul")
+ffi = submodule("_ffi")
 NAMES = ["h"] + GRAD_NAMES
 # ceilings on the fraction of elements of a tensor outside the literal bound, fast kernels (measured: bf16 h, dv 1 %,
 # dq, dk 3-4 %, df, di 4-8 %; fp16 below 1 %)
 CEILING = {torch.bfloat16: 0.12, torch.float16: 0.02}
 
 
-def run_gpu(q, k, v, f, i, dh, precise):
+def run_gpu(q, k, v, f, i, dh, precise, chunk_len=0):
+    """``chunk_len``: 0 = the library's default for the shape, > 0 forces that chunk length (a multiple of 128)."""
     dev = [x.cuda() for x in (q, k, v, f, i, dh)]
-    h, m, b, saved = mm.mlstm_forward_save_hip(*dev[:5], precise=precise)
-    grads = mm.mlstm_backward_saved_hip(dev[5], *dev[:5], h, m, b, saved, precise=precise)
+    ffi.set_chunk_length(chunk_len)
+    try:
+        h, m, b, saved = mm.mlstm_forward_save_hip(*dev[:5], precise=precise)
+        grads = mm.mlstm_backward_saved_hip(dev[5], *dev[:5], h, m, b, saved, precise=precise)
+    finally:
+        ffi.set_chunk_length(0)
     torch.cuda.synchronize()
     return [h, *grads]
 
@@ -50,6 +56,11 @@ def test_thirty_seeds_fast_emulated_precise(dtype):
         emu = O.mlstm_rounded_weights_dense(dh, q, k, v, f, i, dtype)
         fast = run_gpu(q, k, v, f, i, dh, False)
         prec = run_gpu(q, k, v, f, i, dh, True)
+        # split mode in chunks of 128 positions (D = 128 and 256; the kernels of D = 64 know no chunks)
+        chunked = run_gpu(q, k, v, f, i, dh, True, chunk_len=128)
+        for n, r_, c_ in zip(NAMES, ref, chunked):
+            cv = literal_violations(c_, r_)[0]
+            assert cv == 0.0, f"split mode in chunks: {n} seed {seed} S={S} D={D}: {cv:.2e} of the elements outside the literal bound"
         for n, r_, e_, a_, p_ in zip(NAMES, ref, emu, fast, prec):
             frac["fast"][n] += literal_violations(a_, r_)[0] / nseeds
             frac["emulated"][n] += literal_violations(e_.to(dtype), r_)[0] / nseeds
@@ -70,7 +81,7 @@ def test_thirty_seeds_fast_emulated_precise(dtype):
 
 def test_headline_shape_two_heads():
     """B4 H8 S4096 D256 bf16 (runs in chunks of 512): the whole batch through the fast kernels, two heads of it against the
-    oracle; the same two heads in split mode at the literal bound."""
+    oracle; the same two heads in split mode (in chunks of 512 as well, with two-term states) at the literal bound."""
     dtype = torch.bfloat16
     B, NH, S, D = 4, 8, 4096, 256
     q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=0, f_mean=3.0)
@@ -90,8 +101,8 @@ def test_headline_shape_two_heads():
 
 
 def test_long_context_shape_one_head():
-    """cfg 5 per head: S = 16384, D = 128, bf16, f ~ N(3,1), i ~ N(-1,1), dh ~ N(0, 0.1) (fast: chunks of 512; split
-    mode: every key tile).  The oracle's S x S matrices are 2 GiB each in float64."""
+    """cfg 5 per head: S = 16384, D = 128, bf16, f ~ N(3,1), i ~ N(-1,1), dh ~ N(0, 0.1) (chunks of 512 in both modes;
+    split mode with two-term states).  The oracle's S x S matrices are 2 GiB each in float64."""
     dtype = torch.bfloat16
     S, D = 16384, 128
     q, k, v, f, i, dh = O.make_inputs(1, 1, S, D, dtype, seed=5, f_mean=3.0, i_mean=-1.0, dh_std=0.1)

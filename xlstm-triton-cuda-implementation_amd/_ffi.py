@@ -15,7 +15,8 @@ _DTYPES = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dtype)",
            -2: "unsupported shape (head dimension / sequence length)",
            -3: "workspace (or saved buffer) too small or of the wrong size",
-           -4: "a kernel's bounded wait expired"}
+           -4: "a kernel's bounded wait expired",
+           -5: "a backward was given a saved buffer written for another shape or setting"}
 
 GATE_FORMS = {"raw": 0, "logsigmoid": 1, "cumsum": 2}   # MLSTM_GATE_RAW / _LOGSIGMOID / _CUMSUM
 

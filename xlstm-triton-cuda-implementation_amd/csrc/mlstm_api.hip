@@ -55,11 +55,24 @@ struct Carver {
 // 16-bit types at D >= 128; a chunk pays D/64 state tiles per row tile and saves the key tiles before the chunk, and the
 // states cost 2 S D^2 flops per head whatever the length.
 int g_chunk_override = 0;   // test aid: > 0 forces this length, < 0 switches chunking off
-int chunk_len_for(int dtype, int D, size_t S, bool precise = false) {
-    // (split mode runs on the generic kernels, which walk every key tile)
-    if (dtype == MLSTM_F32 || !(D == 128 || D == 256) || mlstm::g_force_generic || g_chunk_override < 0 || precise) return 0;
+int chunk_len_for(int dtype, int D, size_t S) {
+    // (the chunk states are formed by 16-bit MFMA products at D = 128 and 256; every tile kernel of those types knows
+    // chunks, the four-wave ones of split mode and of the test switch included)
+    if (dtype == MLSTM_F32 || !(D == 128 || D == 256) || g_chunk_override < 0) return 0;
     if (g_chunk_override > 0) return S > (size_t)g_chunk_override ? g_chunk_override : 0;
     return S >= 1024 ? 512 : 0;   // (below two full chunks the state pass costs more than the skipped key tiles)
+}
+
+// What mlstm_forward_save_* writes at the head of `saved` and mlstm_backward_saved_* checks on the device (no host
+// round trip): shape, types and the process-wide settings the two calls must agree on.
+constexpr size_t SAVED_HEADER_BYTES = 256;
+struct SavedHeader { int v[8]; };   // magic, BH, S, D, dtype argument, chunk length, kernel switch, states per head
+constexpr int SAVED_MAGIC = 0x4d4c5356;   // "MLSV"
+__global__ void saved_header_write(int* dst, SavedHeader hd) {
+    if (threadIdx.x < 8) dst[threadIdx.x] = hd.v[threadIdx.x];
+}
+__global__ void saved_header_check(const int* src, SavedHeader hd, int* err) {
+    if (threadIdx.x < 8 && src[threadIdx.x] != hd.v[threadIdx.x]) atomicOr(err, 2);
 }
 
 struct Sizes {
@@ -69,27 +82,30 @@ struct Sizes {
     // chunked forward: per-chunk sums (fp32), matrix states (element type), vector states
     size_t n_states(int L) const { return L > 0 && S > (size_t)L ? (S - 1) / L : 0; }
     size_t chunk_states(int dtype) const {
-        const size_t n = n_states(chunk_len_for(dtype, (int)D, S, precise));
-        return up256(BH * n * D * D * 4) + up256(BH * n * D * D * el) + up256(BH * n * D * 4);
+        const size_t n = n_states(chunk_len_for(dtype, (int)D, S));
+        return up256(BH * n * D * D * 4) + up256(BH * n * D * D * el * parts()) + up256(BH * n * D * 4);
     }
     int dtype_code = MLSTM_F32;
     // layouts of the caller's tensors (dense unless an _lx entry point says otherwise): q, k, v and their gradients;
     // h and dh; the gates and their gradients; and what f holds
     Lay la{}, lb{}, lg{};
     int gate_form = MLSTM_GATE_RAW;
-    bool precise = false;   // split mode (MLSTM_PRECISE): no chunks, and the low-order part of h travels to the backward
-    int chunk_len() const { return chunk_len_for(dtype_code, (int)D, S, precise); }
-    size_t states_t() const { return up256(BH * n_states(chunk_len()) * D * D * el); }   // value-major copy for the dQ pass
+    bool precise = false;   // split mode (MLSTM_PRECISE): states as two terms, and the low-order part of h travels to the backward
+    size_t parts() const { return precise ? 2 : 1; }   // terms per matrix state: hi, and lo directly behind it
+    int chunk_len() const { return chunk_len_for(dtype_code, (int)D, S); }
+    size_t state_elems() const { return BH * n_states(chunk_len()) * D * D; }             // one term of one set of states
+    size_t states_t() const { return up256(state_elems() * el * parts()); }               // value-major copy for the dQ pass
     size_t saved_vec() const { return up256(BH * n_states(chunk_len()) * D * 4); }
     size_t h_lo() const { return precise ? up256(BH * S * D * el) : 0; }
-    // the column kernel runs in chunks too when it is the 16x16 one (the generic kernels know no chunks), and only for
-    // lengths at which the eight-wave row kernel, which leaves the far row sums, is sure to have run
+    // the column kernel runs in chunks too, for lengths at which the row kernel, which leaves the far row sums, is sure to
+    // have run in chunks
     bool col_chunks() const { return n_states(chunk_len()) > 0 && NG <= 1024; }
     // row partials of dD per position: one per key tile at or before it, in chunks one per key tile of its own chunk
     size_t row_slices() const { return col_chunks() ? (size_t)chunk_len() / 64 : NG; }
-    // what the backward reuses of the forward: in chunks the value-major states, the vector states and the gate
+    // what the backward reuses of the forward: a header, in chunks the value-major states, the vector states and the gate
     // pre-pass; in split mode h - (h rounded to the element type)
-    size_t saved() const { return precise ? h_lo() : (n_states(chunk_len()) ? states_t() + saved_vec() + gates() : 0); }
+    size_t saved_chunk() const { return n_states(chunk_len()) ? states_t() + saved_vec() + gates() : 0; }
+    size_t saved() const { return saved_chunk() + h_lo() > 0 ? SAVED_HEADER_BYTES + saved_chunk() + h_lo() : 0; }
     // fp32 at head dimensions of 256 and more: the matmul form's entry points run on the scan form's kernels (the same
     // function; the tile kernels' accumulators and LDS stages end at D = 128 in fp32)
     bool scan_engine() const { return dtype_code == MLSTM_F32 && D >= 256; }
@@ -239,7 +255,7 @@ int arm_row_args(RowArgs& a) {
 // the first Sizes::fwd() bytes of every workspace
 struct FwdWs {
     double* G2; float *alpha2, *beta2, *ek2, *amax2, *mw, *bw;
-    int L; size_t ncs; float* dC; char* Cst; float* Nst;
+    int L; size_t ncs; float* dC; char* Cst; char* Cst_lo; float* Nst;
     FwdWs(char* ws, const Sizes& z, int dtype, int D) {
         Carver c{ws, 0};
         G2 = c.take<double>(z.BH * z.NG);
@@ -252,7 +268,8 @@ struct FwdWs {
         L = z.chunk_len();
         ncs = z.n_states(L);
         dC = c.take<float>(z.BH * ncs * z.D * z.D);
-        Cst = c.take<char>(z.BH * ncs * z.D * z.D * z.el);
+        Cst = c.take<char>(z.BH * ncs * z.D * z.D * z.el * z.parts());
+        Cst_lo = z.precise ? Cst + z.BH * ncs * z.D * z.D * z.el : nullptr;
         Nst = c.take<float>(z.BH * ncs * z.D);
     }
     // the gate pre-pass in a buffer of its own (Sizes::gates() bytes) instead of the workspace
@@ -266,12 +283,37 @@ struct FwdWs {
     }
 };
 
-// states at the chunk ends of a long sequence (both layouts when CstT is given)
+// The parts of a `saved` buffer (Sizes::saved() bytes)
+struct SavedView {
+    int* header; char* CstT = nullptr; float* Nst = nullptr; char* gates = nullptr; char* h_lo = nullptr;
+    SavedView(char* sv, const Sizes& z) {
+        header = reinterpret_cast<int*>(sv);
+        char* p = sv + SAVED_HEADER_BYTES;
+        if (z.saved_chunk() > 0) {
+            CstT = p; p += z.states_t();
+            Nst = reinterpret_cast<float*>(p); p += z.saved_vec();
+            gates = p; p += z.gates();
+        }
+        if (z.precise) h_lo = p;
+    }
+};
+SavedHeader saved_header_of(const Sizes& z) {
+    return SavedHeader{{SAVED_MAGIC, (int)z.BH, (int)z.S, (int)z.D, z.dtype_code | (z.precise ? MLSTM_PRECISE : 0), z.chunk_len(),
+                        mlstm::g_force_generic ? 1 : 0, (int)z.n_states(z.chunk_len())}};
+}
+
+// states at the chunk ends of a long sequence (both layouts when CstT is given; split mode: each as two terms, the
+// second directly behind the first)
 int chunk_states_impl(const void* k, const void* v, const FwdWs& w, bool key_major, void* CstT, float* Nst, const Sizes& z, int D, int dtype,
                       hipStream_t st) {
     ChunkArgs ca{k, v, w.alpha2, w.beta2, w.G2, w.dC, Nst, key_major ? w.Cst : nullptr, CstT, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs,
                  0, nullptr, nullptr};
     ca.lk = ca.lv = z.la;
+    ca.precise = z.precise ? 1 : 0;
+    if (z.precise) {
+        ca.Cst_lo = key_major ? w.Cst_lo : nullptr;
+        ca.CstT_lo = CstT ? static_cast<char*>(CstT) + z.state_elems() * z.el : nullptr;
+    }
     Timed t(MLSTM_K_CHUNK_STATES, st);
     return launch_chunk_states(dtype, D, ca, st);
 }
@@ -341,7 +383,7 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
     if (ncs > 0) {   // long sequence: the states at the chunk ends first, then every row tile stays inside its chunk
         float* Nst = Nst_ext ? Nst_ext : w.Nst;
         if (int e = chunk_states_impl(k, v, w, true, CstT, Nst, z, D, dtype, st)) return e;
-        a.chunk_len = w.L; a.n_states = (int)ncs; a.Cst = w.Cst; a.Nst = Nst;
+        a.chunk_len = w.L; a.n_states = (int)ncs; a.Cst = w.Cst; a.Cst_lo = w.Cst_lo; a.Nst = Nst;
     }
     int rc;
     {
@@ -366,7 +408,7 @@ int mlstm_force_generic_kernels(int on) {
 
 int mlstm_chunk_length_for(int S, int D, int dtype) {
     if (S <= 0 || D <= 0 || !good_dtype_arg(dtype)) return 0;
-    return chunk_len_for(dtype & ~MLSTM_PRECISE, D, (size_t)S, precise_of(dtype));
+    return chunk_len_for(dtype & ~MLSTM_PRECISE, D, (size_t)S);
 }
 
 int mlstm_set_chunk_length(int length) {
@@ -396,7 +438,7 @@ int mlstm_kernel_error(void) {
         const int zero = 0;
         e = hipMemcpy(word, &zero, sizeof(int), hipMemcpyHostToDevice);
         if (e != hipSuccess) return (int)e;
-        return MLSTM_EKERNEL;
+        return (value & 1) ? MLSTM_EKERNEL : MLSTM_ESAVED;
     }
     return 0;
 }
@@ -516,13 +558,12 @@ int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const voi
     if (z.saved() > 0 && (!saved || saved_bytes != z.saved())) return MLSTM_EWORKSPACE;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
-    char* sv = z.saved() > 0 ? (char*)saved : nullptr;
-    if (z.precise)   // split mode: what the backward reuses is the low-order part of h
-        return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, sv);
+    if (z.saved() == 0) return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
+    SavedView sv((char*)saved, z);
+    hipLaunchKernelGGL(saved_header_write, dim3(1), dim3(64), 0, st, sv.header, saved_header_of(z));
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                        nullptr, nullptr, nullptr, sv, sv ? reinterpret_cast<float*>(sv + z.states_t()) : nullptr,
-                        sv ? sv + z.states_t() + z.saved_vec() : nullptr);
+                        nullptr, nullptr, nullptr, sv.CstT, sv.Nst, sv.gates, sv.h_lo);
 }
 
 int mlstm_forward_gated_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
@@ -567,25 +608,36 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* colsum = c.take<float>(z.BH * z.S);
     float* rowpart = c.take<float>(z.BH * z.row_slices() * z.S);
     FwdWs w(ws, z, dtype, D);
-    char* CstT = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);
+    char* CstT = c.take<char>(z.state_elems() * z.el * z.parts());
     const float* Nst = w.Nst;
     const bool reuse = saved && w.ncs > 0;
-    if (reuse) {   // the forward's states (value-major matrices, then the vectors) and its gate pre-pass
-        CstT = const_cast<char*>(saved);
-        Nst = reinterpret_cast<const float*>(saved + z.states_t());
-        w.gates_at(const_cast<char*>(saved) + z.states_t() + z.saved_vec(), z);
+    const void* h_lo = nullptr;   // split mode: the low-order part of h, from the forward (saved) or from a recomputation
+    if (saved) {
+        SavedView sv(const_cast<char*>(saved), z);
+        // the header is compared on the device: a buffer written for another shape, type or setting (chunk length, kernel
+        // switch) sets bit 1 of the error word, which mlstm_kernel_error reports
+        int* err = nullptr;
+        if (int rc = symbols_of_current_device(nullptr, &err)) return rc;
+        hipLaunchKernelGGL(saved_header_check, dim3(1), dim3(64), 0, st, sv.header, saved_header_of(z), err);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+        if (reuse) {   // the forward's states (value-major matrices, then the vectors) and its gate pre-pass
+            CstT = sv.CstT;
+            Nst = sv.Nst;
+            w.gates_at(sv.gates, z);
+        }
+        h_lo = sv.h_lo;
     }
-    char* Ev = c.take<char>(z.BH * w.ncs * z.D * z.D * z.el);    // reverse states, value-major
+    char* Ev = c.take<char>(z.state_elems() * z.el * z.parts());    // reverse states, value-major
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs);
     char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
+    const size_t lo_off = z.state_elems() * z.el;   // split mode: a set of states is [hi | lo]
     const bool col_chunks = z.col_chunks();
 
     float *alpha2, *beta2, *mm, *bb, *ek2, *amax2; double* G2;
     // Split mode needs h beyond the element type's precision for dh . h: either the forward left the low-order part
     // (saved), or the forward is run again here
-    const void* h_lo = z.precise ? saved : nullptr;
     const bool have_fwd = h && m && b && (!z.precise || h_lo);
     Lay lh = z.lb;   // layout of the forward output the dQ pass reads
     if (have_fwd) {
@@ -619,7 +671,10 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ra.BH = (int)z.BH; ra.S = (int)z.S; ra.NG = (int)z.NG;
     ra.precise = z.precise ? 1 : 0; ra.Hin_lo = h_lo;
     if (int rc = arm_row_args(ra)) return rc;
-    if (w.ncs > 0) { ra.chunk_len = w.L; ra.n_states = (int)w.ncs; ra.Cst = CstT; ra.Nst = Nst; ra.Qrow = q; ra.rowinter = rowinter; }
+    if (w.ncs > 0) {
+        ra.chunk_len = w.L; ra.n_states = (int)w.ncs; ra.Cst = CstT; ra.Cst_lo = z.precise ? CstT + lo_off : nullptr; ra.Nst = Nst; ra.Qrow = q;
+        ra.rowinter = rowinter;
+    }
     {
         Timed t(MLSTM_K_ROW_DQ, st);
         if (int rc = launch_row_best(1, dtype, D, ra, st)) return rc;
@@ -631,8 +686,12 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         Timed t(MLSTM_K_CHUNK_STATES, st);
         ChunkArgs ra2{q, dh, alpha2, beta2, G2, w.dC, gvec, nullptr, Ev, (int)z.BH, (int)z.S, (int)z.NG, w.L, (int)w.ncs, 1, inv_n, dbuf};
         ra2.lk = z.la; ra2.lv = z.lb;
+        ra2.precise = z.precise ? 1 : 0;
+        ra2.CstT_lo = z.precise ? Ev + lo_off : nullptr;
         if (int e = launch_chunk_states(dtype, D, ra2, st)) return e;
-        if (int e = launch_anchor(dtype, D, CstT, Ev, Nst, gvec, anchor, (int)z.BH, (int)w.ncs, st)) return e;   // (both value-major)
+        if (int e = launch_anchor(dtype, D, CstT, Ev, z.precise ? CstT + lo_off : nullptr, z.precise ? Ev + lo_off : nullptr, Nst, gvec, anchor,
+                                  (int)z.BH, (int)w.ncs, st))
+            return e;   // (both value-major)
     }
     ColArgs ca{};
     ca.la = z.la; ca.lb = z.lb;
@@ -640,7 +699,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     ca.alpha2 = alpha2; ca.beta2 = beta2; ca.G2 = G2; ca.inv_n = inv_n; ca.db = dbuf;
     ca.BH = (int)z.BH; ca.S = (int)z.S; ca.NG = (int)z.NG;
     ca.precise = z.precise ? 1 : 0; ca.RS = (int)z.row_slices();
-    if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ev = Ev; ca.gvec = gvec; }
+    if (col_chunks) { ca.chunk_len = w.L; ca.n_states = (int)w.ncs; ca.Ev = Ev; ca.Ev_lo = z.precise ? Ev + lo_off : nullptr; ca.gvec = gvec; }
     {
         Timed t(MLSTM_K_COL, st);
         if (int rc = launch_col_best(dtype, D, ca, st)) return rc;

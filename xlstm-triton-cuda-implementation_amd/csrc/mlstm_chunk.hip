@@ -28,12 +28,14 @@ namespace mlstm {
 // state row PERM16(u): the two middle groups of four swap places.
 __device__ __forceinline__ int perm16(int u) { return (u & ~12) | ((u & 4) << 1) | ((u & 8) >> 1); }
 
-template <typename T, int D>
+// STRICT: split mode, the weighted V rows go to LDS as two tiles, hi and lo (ChunkArgs::precise)
+template <typename T, int D, bool STRICT = false>
 struct ChunkCfg {
     static constexpr int VW = 128;                                  // value columns per workgroup
     static constexpr int STAGES = 2;                                // LDS stages: the tile worked on and the next one
     static constexpr int RSETS = 3;                                 // register sets: tiles in flight from memory
-    static constexpr size_t K_BYTES = (size_t)GRAN * D * sizeof(T), V_BYTES = (size_t)GRAN * VW * sizeof(T);
+    static constexpr size_t K_BYTES = (size_t)GRAN * D * sizeof(T), V_TILE = (size_t)GRAN * VW * sizeof(T);
+    static constexpr size_t V_BYTES = (STRICT ? 2 : 1) * V_TILE;    // per stage: the hi tile, then the lo tile
     static constexpr size_t TILE_BYTES = STAGES * (K_BYTES + V_BYTES);   // plus one float per position of the chunk
     static constexpr int MAX_L = (int)((160 * 1024 - TILE_BYTES) / (2 * sizeof(float))) / 128 * 128;
 };
@@ -64,11 +66,11 @@ template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
 
 // NTT: tiles per chunk as a compile-time constant (the tile loop is then straight-line code), or 0 for any chunk length
-template <typename T, int D, int NTT>
+template <typename T, int D, int NTT, bool STRICT>
 __global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using R = Tr<T>;
-    using Cfg = ChunkCfg<T, D>;
+    using Cfg = ChunkCfg<T, D, STRICT>;
     typedef typename R::frag frag;
     static_assert(R::HALF && (D == 128 || D == 256), "16-bit types, D = 128 or 256");
     constexpr int VW = Cfg::VW, VH = D / VW, MB = D / 128, NB = VW / 32, KW = R::KW, ST = Cfg::STAGES;
@@ -170,8 +172,15 @@ __global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
             float x[8];
             unpack8<T>(vset[P][it], x);
             Pair out;
-            out.lo = R::cvt4(f32x4{x[0] * w, x[1] * w, x[2] * w, x[3] * w});
-            out.hi = R::cvt4(f32x4{x[4] * w, x[5] * w, x[6] * w, x[7] * w});
+            if constexpr (STRICT) {   // the weighted row as two terms: what rounding to the element type loses goes to the lo tile
+                Pair rest;
+                R::cvt4_split(f32x4{x[0] * w, x[1] * w, x[2] * w, x[3] * w}, out.lo, rest.lo);
+                R::cvt4_split(f32x4{x[4] * w, x[5] * w, x[6] * w, x[7] * w}, out.hi, rest.hi);
+                *reinterpret_cast<Pair*>(vs + (j % ST) * Cfg::V_BYTES + Cfg::V_TILE + ZV::off(row, 8 * vch)) = rest;
+            } else {
+                out.lo = R::cvt4(f32x4{x[0] * w, x[1] * w, x[2] * w, x[3] * w});
+                out.hi = R::cvt4(f32x4{x[4] * w, x[5] * w, x[6] * w, x[7] * w});
+            }
             *reinterpret_cast<Pair*>(vs + (j % ST) * Cfg::V_BYTES + ZV::off(row, 8 * vch)) = out;
         }
     };
@@ -306,7 +315,8 @@ __global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
         // the operand reads of a contraction step run one step ahead of its MFMAs (read, wait, multiply in turns left the
         // matrix unit idle for an LDS round trip per step: 3000 cycles per tile for 1024 of MFMAs, measured)
         constexpr int NSTEP = GRAN / KW;
-        frag af[2][MB], bf[2][NB];
+        frag af[2][MB], bf[2][NB], bl[STRICT ? NB : 1];
+        const T* vl = reinterpret_cast<const T*>(vs + (t % ST) * Cfg::V_BYTES + Cfg::V_TILE);   // (split mode: the lo tile)
         auto rd = [&](int s) __attribute__((always_inline)) {
 #pragma unroll
             for (int mb = 0; mb < MB; mb++) af[s & 1][mb] = krd.read(kt, KW * s, mb);
@@ -316,11 +326,23 @@ __global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
         rd(0);
 #pragma unroll
         for (int s = 0; s < NSTEP; s++) {
+            // (split mode: the lo fragments of this step are single-buffered -- a second set does not fit the registers at
+            // D = 256 -- and requested here, behind the MFMAs on the hi fragments)
+            if constexpr (STRICT) {
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) bl[nb] = vrd.read(vl, KW * s, nb);
+            }
             if (s + 1 < NSTEP) rd(s + 1);
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
                 for (int nb = 0; nb < NB; nb++) R::mma(acc[mb][nb], af[s & 1][mb], bf[s & 1][nb]);
+            if constexpr (STRICT) {
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++) R::mma(acc[mb][nb], af[s & 1][mb], bl[nb]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -382,8 +404,15 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
             typedef typename Tr<T>::vec4 V4;
             struct Pair { V4 lo, hi; };
             Pair o;
-            o.lo = Tr<T>::cvt4(run0);
-            o.hi = Tr<T>::cvt4(run1);
+            if (a.Cst_lo) {   // split mode: the state as two terms
+                Pair rest;
+                Tr<T>::cvt4_split(run0, o.lo, rest.lo);
+                Tr<T>::cvt4_split(run1, o.hi, rest.hi);
+                *reinterpret_cast<Pair*>(reinterpret_cast<T*>(a.Cst_lo) + (dst - reinterpret_cast<T*>(a.Cst)) + (size_t)c * D * D) = rest;
+            } else {
+                o.lo = Tr<T>::cvt4(run0);
+                o.hi = Tr<T>::cvt4(run1);
+            }
             *reinterpret_cast<Pair*>(dst + (size_t)c * D * D) = o;
         }
         if (vec) {
@@ -399,8 +428,9 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
 // kernel, like the untransposed states.
 template <typename T, int D>
 __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
-    __shared__ __attribute__((aligned(16))) T tile[64][64 + 8];
+    __shared__ __attribute__((aligned(16))) T tile[2][64][64 + 8];   // [hi | lo (split mode)]
     const int bh = blockIdx.y, tid = threadIdx.x;
+    const bool split = a.CstT_lo != nullptr;
     const int vb = blockIdx.x % (D / 64), kb = blockIdx.x / (D / 64);
     const int vl = tid & 63, kq = tid >> 6;
     const size_t poff = (size_t)bh * a.NG * GRAN, goff = (size_t)bh * a.NG;
@@ -431,41 +461,66 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
             for (int e = 0; e < 8; e++) d[e] = src[(size_t)(64 * kb + 8 * (kq + 4 * g) + e) * D];
             run[g] = run[g] * gam + d;
             if (a.Cst) {   // key-major copy: lanes of a wave hold consecutive values of one key, 128 bytes per store
-                T* kd = reinterpret_cast<T*>(a.Cst) + ((size_t)bh * a.NCS + c) * D * D + 64 * vb + vl;
+                const size_t koff = ((size_t)bh * a.NCS + c) * D * D + 64 * vb + vl;
+                T* kd = reinterpret_cast<T*>(a.Cst) + koff;
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int k = 64 * kb + 8 * (kq + 4 * g) + e;
-                    kd[(size_t)((k & ~15) | perm16(k & 15)) * D] = (T)run[g][e];
+                    const T hi = (T)run[g][e];
+                    kd[(size_t)((k & ~15) | perm16(k & 15)) * D] = hi;
+                    if (a.Cst_lo) (reinterpret_cast<T*>(a.Cst_lo) + koff)[(size_t)((k & ~15) | perm16(k & 15)) * D] = (T)(run[g][e] - (float)hi);
                 }
             }
             typedef typename Tr<T>::vec4 V4;
             struct Pair { V4 lo, hi; };
             Pair o;
-            o.lo = Tr<T>::cvt4(__builtin_shufflevector(run[g], run[g], 0, 1, 2, 3));
-            o.hi = Tr<T>::cvt4(__builtin_shufflevector(run[g], run[g], 4, 5, 6, 7));
-            *reinterpret_cast<Pair*>(&tile[vl][8 * (kq + 4 * g)]) = o;
+            if (split) {   // the state as two terms: the second holds what rounding to the element type loses
+                Pair rest;
+                Tr<T>::cvt4_split(__builtin_shufflevector(run[g], run[g], 0, 1, 2, 3), o.lo, rest.lo);
+                Tr<T>::cvt4_split(__builtin_shufflevector(run[g], run[g], 4, 5, 6, 7), o.hi, rest.hi);
+                *reinterpret_cast<Pair*>(&tile[1][vl][8 * (kq + 4 * g)]) = rest;
+            } else {
+                o.lo = Tr<T>::cvt4(__builtin_shufflevector(run[g], run[g], 0, 1, 2, 3));
+                o.hi = Tr<T>::cvt4(__builtin_shufflevector(run[g], run[g], 4, 5, 6, 7));
+            }
+            *reinterpret_cast<Pair*>(&tile[0][vl][8 * (kq + 4 * g)]) = o;
         }
         __syncthreads();
-        const uint4 p0 = *reinterpret_cast<const uint4*>(&tile[orow][16 * opiece]), p1 = *reinterpret_cast<const uint4*>(&tile[orow][16 * opiece + 8]);
+        const uint4 p0 = *reinterpret_cast<const uint4*>(&tile[0][orow][16 * opiece]), p1 = *reinterpret_cast<const uint4*>(&tile[0][orow][16 * opiece + 8]);
         *reinterpret_cast<uint4*>(dst + (size_t)c * D * D) = p0;
         *reinterpret_cast<uint4*>(dst + (size_t)c * D * D + 8) = p1;
+        if (split) {
+            T* dlo = reinterpret_cast<T*>(a.CstT_lo) + (dst - reinterpret_cast<T*>(a.CstT));
+            *reinterpret_cast<uint4*>(dlo + (size_t)c * D * D) = *reinterpret_cast<const uint4*>(&tile[1][orow][16 * opiece]);
+            *reinterpret_cast<uint4*>(dlo + (size_t)c * D * D + 8) = *reinterpret_cast<const uint4*>(&tile[1][orow][16 * opiece + 8]);
+        }
         __syncthreads();
     }
 }
 
-template <typename T, int D>
-static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
-    using Cfg = ChunkCfg<T, D>;
+template <typename T, int D, bool STRICT>
+static int launch_chunk_sum(const ChunkArgs& a, hipStream_t st) {
+    using Cfg = ChunkCfg<T, D, STRICT>;
     if (a.L > Cfg::MAX_L) return MLSTM_ESHAPE;
     const dim3 grid(a.BH * a.NCS * (D / Cfg::VW));
     const size_t lds = Cfg::TILE_BYTES + 2 * (size_t)a.L * sizeof(float);
-    if (a.L == 8 * GRAN) {   // the default chunk length
-        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 8>>(160 * 1024); e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 8>), grid, dim3(512), lds, st, a);
+    // (the unrolled variant of split mode at D = 256 does not fit the 256 registers of a wave and would spill)
+    constexpr bool UNROLLED_FITS = !(STRICT && D == 256);
+    if (UNROLLED_FITS && a.L == 8 * GRAN) {   // the default chunk length
+        constexpr int NTT = UNROLLED_FITS ? 8 : 0;
+        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, NTT, STRICT>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, NTT, STRICT>), grid, dim3(512), lds, st, a);
     } else {
-        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 0>>(160 * 1024); e != hipSuccess) return (int)e;
-        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 0>), grid, dim3(512), lds, st, a);
+        if (hipError_t e = lds_limit_once<chunk_sum_kernel<T, D, 0, STRICT>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_sum_kernel<T, D, 0, STRICT>), grid, dim3(512), lds, st, a);
     }
+    return 0;
+}
+
+template <typename T, int D>
+static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
+    if (a.precise && ((a.Cst && !a.Cst_lo) || (a.CstT && !a.CstT_lo))) return MLSTM_EINVAL;
+    if (int rc = a.precise ? launch_chunk_sum<T, D, true>(a, st) : launch_chunk_sum<T, D, false>(a, st)) return rc;
     // one carry kernel: the value-major one writes both layouts and the vector states
     if (a.CstT) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D>), dim3((D / 64) * (D / 64), a.BH), dim3(256), 0, st, a);
     else hipLaunchKernelGGL((chunk_carry_kernel<T, D>), dim3(D * D / 8 / 256, a.BH), dim3(256), 0, st, a);
@@ -476,16 +531,21 @@ static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
 // contracted with the reverse state, <C~_c, E_c> + n~_c . g_c.  Rounding errors of the two matrices' 16-bit entries
 // average out over the D^2 products.
 template <typename T>
-__global__ __launch_bounds__(1024) void anchor_kernel(const T* __restrict__ A, const T* __restrict__ B, const float* __restrict__ va,
-                                                     const float* __restrict__ vb, float* __restrict__ anchor, int D, int NCS) {
+__global__ __launch_bounds__(1024) void anchor_kernel(const T* __restrict__ A, const T* __restrict__ B, const T* __restrict__ Al,
+                                                     const T* __restrict__ Bl, const float* __restrict__ va, const float* __restrict__ vb,
+                                                     float* __restrict__ anchor, int D, int NCS) {
     __shared__ float part[16];
     const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
     const size_t base = ((size_t)bh * NCS + c) * D * D;
     typedef typename Tr<T>::frag V8;
     float acc = 0.f;
     for (int e = 8 * tid; e < D * D; e += 8 * 1024) {
-        const f32x8 x = __builtin_convertvector(*reinterpret_cast<const V8*>(A + base + e), f32x8);
-        const f32x8 y = __builtin_convertvector(*reinterpret_cast<const V8*>(B + base + e), f32x8);
+        f32x8 x = __builtin_convertvector(*reinterpret_cast<const V8*>(A + base + e), f32x8);
+        f32x8 y = __builtin_convertvector(*reinterpret_cast<const V8*>(B + base + e), f32x8);
+        if (Al) {   // split mode: both states as hi + lo (the sums are exact in fp32: 8 + 8 significant bits at most)
+            x += __builtin_convertvector(*reinterpret_cast<const V8*>(Al + base + e), f32x8);
+            y += __builtin_convertvector(*reinterpret_cast<const V8*>(Bl + base + e), f32x8);
+        }
         acc += ((x[0] * y[0] + x[1] * y[1]) + (x[2] * y[2] + x[3] * y[3])) + ((x[4] * y[4] + x[5] * y[5]) + (x[6] * y[6] + x[7] * y[7]));
     }
     if (tid < D) acc += va[((size_t)bh * NCS + c) * D + tid] * vb[((size_t)bh * NCS + c) * D + tid];
@@ -501,11 +561,15 @@ __global__ __launch_bounds__(1024) void anchor_kernel(const T* __restrict__ A, c
     }
 }
 
-int launch_anchor(int dtype, int D, const void* A, const void* B, const float* va, const float* vb, float* anchor, int BH, int NCS, hipStream_t st) {
+int launch_anchor(int dtype, int D, const void* A, const void* B, const void* A_lo, const void* B_lo, const float* va, const float* vb,
+                  float* anchor, int BH, int NCS, hipStream_t st) {
+    if ((A_lo == nullptr) != (B_lo == nullptr)) return MLSTM_EINVAL;
     if (dtype == MLSTM_BF16)
-        hipLaunchKernelGGL(anchor_kernel<__bf16>, dim3(NCS, BH), dim3(1024), 0, st, (const __bf16*)A, (const __bf16*)B, va, vb, anchor, D, NCS);
+        hipLaunchKernelGGL(anchor_kernel<__bf16>, dim3(NCS, BH), dim3(1024), 0, st, (const __bf16*)A, (const __bf16*)B, (const __bf16*)A_lo,
+                           (const __bf16*)B_lo, va, vb, anchor, D, NCS);
     else if (dtype == MLSTM_F16)
-        hipLaunchKernelGGL(anchor_kernel<_Float16>, dim3(NCS, BH), dim3(1024), 0, st, (const _Float16*)A, (const _Float16*)B, va, vb, anchor, D, NCS);
+        hipLaunchKernelGGL(anchor_kernel<_Float16>, dim3(NCS, BH), dim3(1024), 0, st, (const _Float16*)A, (const _Float16*)B,
+                           (const _Float16*)A_lo, (const _Float16*)B_lo, va, vb, anchor, D, NCS);
     else return MLSTM_ESHAPE;
     return (int)hipGetLastError();
 }

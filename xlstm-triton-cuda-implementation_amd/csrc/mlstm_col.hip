@@ -13,6 +13,11 @@
 // Column sums of dD (= dI) stay in registers for the whole kernel; row sums leave the kernel as one partial per
 // (key tile, query) and are added up by the dF pass, so rows and columns are sums of the very same fp32 products
 // and the cancellation in dF = sigmoid(-f) * cumsum(col - row) stays exact to fp32 round-off.
+//
+// Long sequences in chunks (ColArgs::chunk_len): the keys walk the query tiles of their own chunk only; what the queries
+// behind the chunk contribute comes through the chunk's reverse state E (value-major, mlstm_chunk.hip) in a state phase
+// ahead of the query loop:  dK_j = w_j (E v_j + g),  dV_j = w_j E^T k_j,  w_j = exp(a_j - A_e), e the chunk's last
+// position, and k_j . dK_j of that part goes into the column sums.  In split mode E comes as two terms, hi + lo.
 #include <mutex>
 #include <type_traits>
 #include "mlstm_device.h"
@@ -30,9 +35,15 @@ struct ColCfg {
     static constexpr size_t G_BYTES = (size_t)GRAN * LDG * sizeof(T);
     // G, W (split mode: and their low-order terms), row-sum scratch.  With the two extra tiles the 16-bit D = 256 case
     // no longer fits two query stages and runs single-staged.
-    static constexpr size_t FIXED_BYTES = (STRICT ? 4 : 2) * G_BYTES + 2 * GRAN * sizeof(float);
+    static constexpr size_t GW_BYTES = (STRICT ? 4 : 2) * G_BYTES;
+    static constexpr size_t FIXED_BYTES = GW_BYTES + 6 * GRAN * sizeof(float);   // + row sums [2][64], far column sums [4][64]
     static constexpr int STAGES = (2 * STAGE_BYTES + FIXED_BYTES + 2048 * sizeof(float) <= 160 * 1024) ? 2 : 1;
     static constexpr size_t LDS_BYTES = STAGES * STAGE_BYTES + FIXED_BYTES;  // plus one float per key tile, appended at launch
+    // In chunks the keys' own K and V tiles lie in LDS during the state phase: in the second stage where there is one;
+    // otherwise K in the (not yet used) G / W area and V in an extra tile between the fixed part and the granule bases
+    static constexpr size_t TILE_BYTES = TILE_ELEMS * sizeof(T);
+    static constexpr size_t EXTRA_CHUNK_BYTES = STAGES == 2 ? 0 : TILE_BYTES;
+    static_assert(STAGES == 2 || GW_BYTES >= TILE_BYTES, "the keys' K tile fits the G / W area");
 };
 
 // Swizzle key of the 16-bit G / W tiles: bits (q>>1)&1 and (q>>2)&3 of the query row.  Phase A writes one chunk of
@@ -64,7 +75,9 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
     T* const Gl = Ws + GRAN * LDG;                                    // split mode: low-order terms of G and W
     T* const Wl = Gl + GRAN * LDG;
     float* const rowtmp = reinterpret_cast<float*>(Gs + (STRICT ? 4 : 2) * GRAN * LDG);  // [2][64]
-    float* const sG = reinterpret_cast<float*>(smem + Cfg::LDS_BYTES);  // granule bases minus this key tile's (see row kernel)
+    float* const cpart = rowtmp + 2 * GRAN;                                               // [4][64]
+    // granule bases minus this key tile's (see row kernel)
+    float* const sG = reinterpret_cast<float*>(smem + Cfg::LDS_BYTES + (a.chunk_len > 0 ? Cfg::EXTRA_CHUNK_BYTES : 0));
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
     const int S = a.S, NG = a.NG;
@@ -110,7 +123,34 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
         }                                                                        \
         rvdma.issue(ST_ROW(st), (it));                                            \
     } while (0)
-    COL_DMA(jt, 0);  // first of all: its latency then overlaps that of the plain loads below
+    // In chunks the keys walk the query tiles of their own chunk only (NGe: one past the last of them)
+    const int tpc = a.chunk_len > 0 ? a.chunk_len / GRAN : 0;
+    const int chunk = a.chunk_len > 0 ? jt / tpc : 0;
+    const int NGe = a.chunk_len > 0 ? ((chunk + 1) * tpc < NG ? (chunk + 1) * tpc : NG) : NG;
+    const bool has_state = a.chunk_len > 0 && chunk < a.n_states;   // (uniform over the workgroup)
+    constexpr int NTL = D / GRAN;   // 64-row tiles of a state
+    T* const Kt = STAGES == 2 ? ST_Q(1) : Gs;
+    T* const Vt = STAGES == 2 ? ST_DH(1) : reinterpret_cast<T*>(smem + Cfg::LDS_BYTES);
+    const size_t sbase = has_state ? ((size_t)bh * a.n_states + chunk) * D * D : 0;
+    const T* const Evc = reinterpret_cast<const T*>(a.Ev) + sbase;
+    const T* const Evl = STRICT ? reinterpret_cast<const T*>(a.Ev_lo) + sbase : nullptr;
+    // state tile tau: split mode hi -> Q slot, lo -> dH slot of stage 0, one tile per round; otherwise tile tau -> slot
+    // tau & 1, the next tile travelling while this one is worked on
+    auto state_issue = [&](int tau) {
+        if constexpr (STRICT) {
+            tdma.issue(ST_Q(0), Evc + (size_t)GRAN * tau * D);
+            tdma.issue(ST_DH(0), Evl + (size_t)GRAN * tau * D);
+        } else {
+            tdma.issue((tau & 1) ? ST_DH(0) : ST_Q(0), Evc + (size_t)GRAN * tau * D);
+        }
+    };
+    if (has_state) {   // (a chunk with a successor is complete: its key tiles have all their rows)
+        tdma.issue(Kt, K + (size_t)GRAN * jt * rsA, ra);
+        tdma.issue(Vt, V + (size_t)GRAN * jt * rsA, ra);
+        state_issue(0);
+    } else {
+        COL_DMA(jt, 0);  // first of all: its latency then overlaps that of the plain loads below
+    }
     {
         const double gj = a.G2[(size_t)bh * a.NG + jt];
         for (int g = threadIdx.x; g < a.NG; g += 256) sG[g] = (float)(a.G2[(size_t)bh * a.NG + g] - gj);
@@ -163,6 +203,109 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
     SwzTransReader<typename std::conditional<FAST_TR, T, __bf16>::type, FAST_TR ? D : 256> trd;
     if constexpr (FAST_TR) trd.init(lane, BOTH_KB ? wave * NXW : 0);
 
+    // ---- state phase (sequences in chunks)
+    // (k_j . dK_j of the state part, the far column sums, stay in cpart[0..63] until the end of the kernel)
+    if (has_state) {
+        constexpr int NGRP = GRAN / KW;
+        const int pe = (chunk + 1) * a.chunk_len - 1;   // the chunk's last position
+        const float bend = a.beta2[poff + pe];
+        const double dG = a.G2[(size_t)bh * a.NG + pe / GRAN] - a.G2[(size_t)bh * a.NG + jt];   // (the keys' granule is jt)
+        float wk[NKB];
+#pragma unroll
+        for (int kb = 0; kb < NKB; kb++) wk[kb] = fast_exp2(a.alpha2[poff + GRAN * jt + 32 * (BOTH_KB ? kb : kbB) + c32] - bend + (float)dG);
+        auto col_block = [&](int x) { return BOTH_KB ? wave * NXW + x : dsel + 2 * x; };
+        auto rd_tr = [&](const T* tile, int tt, int x) {
+            if constexpr (FAST_TR) return trd.read(tile, KW * tt, BOTH_KB ? x : col_block(x));
+            else return swz_frag_transposed<T, D>(tile, KW * tt, 32 * col_block(x), lane);
+        };
+#pragma unroll
+        for (int tau = 0; tau < NTL; tau++) {
+            dma_wait();
+            __syncthreads();   // tile tau (and, the first time, the keys' K and V) have landed
+            const T* th = STRICT ? ST_Q(0) : ((tau & 1) ? ST_DH(0) : ST_Q(0));
+            const T* tl = ST_DH(0);
+            if constexpr (!STRICT) { if (tau + 1 < NTL) state_issue(tau + 1); }
+            // dK: contraction over this tile's 64 rows (values 64 tau ..), the wave's columns of the state
+#pragma unroll
+            for (int tt = 0; tt < NGRP; tt++) {
+                frag vB[NKB], ea[NXW], el[STRICT ? NXW : 1];
+#pragma unroll
+                for (int kb = 0; kb < NKB; kb++) vB[kb] = swz_frag_rowmajor<T, D>(Vt, 32 * (BOTH_KB ? kb : kbB) + c32, NGRP * tau + tt, h);
+#pragma unroll
+                for (int x = 0; x < NXW; x++) {
+                    ea[x] = rd_tr(th, tt, x);
+                    if constexpr (STRICT) el[x] = rd_tr(tl, tt, x);
+                }
+#pragma unroll
+                for (int x = 0; x < NXW; x++)
+#pragma unroll
+                    for (int kb = 0; kb < NKB; kb++) {
+                        R::mma(dkacc[kb][x], ea[x], vB[kb]);
+                        if constexpr (STRICT) R::mma(dkacc[kb][x], el[x], vB[kb]);
+                    }
+            }
+            // dV: the wave's own rows of the state, if this tile holds them, contracted over the whole key index
+#pragma unroll
+            for (int x = 0; x < NXW; x++) {
+                const int r0v = 32 * col_block(x);
+                if (r0v / GRAN != tau) continue;
+                const int rl = r0v % GRAN + c32;
+                // (16-bit states keep their rows in the contraction order of the transposing reads, see mlstm_chunk.hip)
+                const int own = R::HALF ? ((rl & ~15) | ((rl & 3) | ((rl & 4) << 1) | ((rl & 8) >> 1))) : rl;
+#pragma unroll
+                for (int t = 0; t < NS; t++) {
+                    frag kB[NKB];
+#pragma unroll
+                    for (int kb = 0; kb < NKB; kb++) kB[kb] = swz_frag_rowmajor<T, D>(Kt, 32 * (BOTH_KB ? kb : kbB) + c32, t, h);
+                    const frag eb = swz_frag_rowmajor<T, D>(th, own, t, h);
+#pragma unroll
+                    for (int kb = 0; kb < NKB; kb++) R::mma(dvacc[kb][x], eb, kB[kb]);
+                    if constexpr (STRICT) {
+                        const frag ebl = swz_frag_rowmajor<T, D>(tl, own, t, h);
+#pragma unroll
+                        for (int kb = 0; kb < NKB; kb++) R::mma(dvacc[kb][x], ebl, kB[kb]);
+                    }
+                }
+            }
+            if constexpr (STRICT) {
+                __syncthreads();   // every wave is done with the tile: the next one may overwrite it
+                if (tau + 1 < NTL) state_issue(tau + 1);
+            }
+        }
+        if constexpr (!STRICT) __syncthreads();   // every wave is done with stage 0
+        COL_DMA(jt, 0);   // the first query tile follows the state into stage 0
+        // the keys' weights, the vector state, and k_j . dK_j for the column sums
+        const float* gv = a.gvec + ((size_t)bh * a.n_states + chunk) * D;
+#pragma unroll
+        for (int kb = 0; kb < NKB; kb++) {
+            float cp = 0.f;
+            const int krow = 32 * (BOTH_KB ? kb : kbB) + c32;
+#pragma unroll
+            for (int x = 0; x < NXW; x++)
+#pragma unroll
+                for (int a4 = 0; a4 < 4; a4++) {
+                    const int d = 32 * col_block(x) + 8 * a4 + 4 * h;
+                    const f32x4 g4v = *reinterpret_cast<const f32x4*>(gv + d);
+                    const char* kp = reinterpret_cast<const char*>(Kt) + Swz<T, D>::off(krow, d & ~(Swz<T, D>::EPC - 1)) + (d & (Swz<T, D>::EPC - 1)) * (int)sizeof(T);
+                    const f32x4 kv = __builtin_convertvector(*reinterpret_cast<const typename R::vec4*>(kp), f32x4);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const float dkv = (dkacc[kb][x][4 * a4 + c] + g4v[c]) * wk[kb];
+                        dkacc[kb][x][4 * a4 + c] = dkv;
+                        dvacc[kb][x][4 * a4 + c] *= wk[kb];
+                        cp += dkv * kv[c];
+                    }
+                }
+            cp = sum_halves(cp);
+            if (h == 0) {
+                cpart[wave * GRAN + krow] = cp;
+                if constexpr (!BOTH_KB) cpart[wave * GRAN + (krow ^ 32)] = 0.f;
+            }
+        }
+        __syncthreads();   // the waves' shares of k . dK lie in LDS (and Kt, in the G / W area, is done with)
+        if (tid < GRAN) cpart[tid] = (cpart[tid] + cpart[GRAN + tid]) + (cpart[2 * GRAN + tid] + cpart[3 * GRAN + tid]);
+    }
+
     // transposing read of the swizzled 16-bit G / W tiles: contraction rows 16t + 8x + 4h + (j>>2), keys 32*kbB + ..
     int gwoff[NKB][2];
     {
@@ -200,7 +343,7 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
             if constexpr (SPREAD) {
                 rvdma.issue(ST_ROW(stn), it + 1);
             } else {
-                if (it + 1 < NG) { if (stage) COL_DMA(it + 1, 0); else COL_DMA(it + 1, 1); }
+                if (it + 1 < NGe) { if (stage) COL_DMA(it + 1, 0); else COL_DMA(it + 1, 1); }
             }
         }
         const T* gq = Q + (size_t)GRAN * (it + 1) * rsA;
@@ -355,18 +498,18 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
                 }
             }
         }
-        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * a.RS + jt) * S + qi0 + tid] = rp0 + rp1;   // (RS == NG: no chunks here)
+        if (tid < GRAN && qi0 + tid < S) a.rowpart[((size_t)bh * a.RS + (a.RS == NG ? jt : jt % a.RS)) * S + qi0 + tid] = rp0 + rp1;
         if constexpr (STAGES == 1) {
             __syncthreads();  // single stage: everyone is done reading before the overwrite, which the next top barrier awaits
-            if (it + 1 < NG) COL_DMA(it + 1, 0);
+            if (it + 1 < NGe) COL_DMA(it + 1, 0);
         }
     };
     // steps whose successor tile exists and is complete spread its copy over their MFMAs; the others copy in one go
-    const int lim = (NG < full_tiles ? NG : full_tiles) - 1;   // last step index that may spread is lim - 1
+    const int lim = (NGe < full_tiles ? NGe : full_tiles) - 1;   // last step index that may spread is lim - 1
     step(std::true_type{}, std::false_type{}, jt);  // the diagonal step skips a block in some waves: it copies in one go
     int it = jt + 1;
     for (; it < lim; it++) step(std::false_type{}, std::true_type{}, it);
-    for (; it < NG; it++) step(std::false_type{}, std::false_type{}, it);
+    for (; it < NGe; it++) step(std::false_type{}, std::false_type{}, it);
 #undef COL_DMA
 #undef ST_Q
 #undef ST_DH
@@ -416,7 +559,7 @@ __global__ __launch_bounds__(256, 1) void col_kernel(ColArgs a) {
         if (c32 == 0) rowtmp[qbA * GRAN + 32 * kbA + 8 * (r >> 2) + 4 * h + (r & 3)] = v;
     }
     __syncthreads();
-    if (tid < GRAN && GRAN * jt + tid < S) a.colsum[hoff + GRAN * jt + tid] = rowtmp[tid] + rowtmp[GRAN + tid];
+    if (tid < GRAN && GRAN * jt + tid < S) a.colsum[hoff + GRAN * jt + tid] = rowtmp[tid] + rowtmp[GRAN + tid] + (has_state ? cpart[tid] : 0.f);
 #endif
 }
 
@@ -428,11 +571,14 @@ static int launch_col_ts(const ColArgs& a, hipStream_t st) {
     static hipError_t attr_rc = hipSuccess;
     std::call_once(once, [&] {
         attr_rc = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                      (int)(Cfg::LDS_BYTES + 2048 * sizeof(float)));
+                                      (int)(Cfg::LDS_BYTES + Cfg::EXTRA_CHUNK_BYTES + 2048 * sizeof(float)));
     });
     if (attr_rc != hipSuccess) return (int)attr_rc;
     if (a.NG > 2048) return MLSTM_ESHAPE;
-    hipLaunchKernelGGL(kern, dim3(a.BH * a.NG), dim3(256), Cfg::LDS_BYTES + (size_t)a.NG * sizeof(float), st, a);
+    if (a.chunk_len > 0 && (a.chunk_len % GRAN != 0 || (a.n_states > 0 && (!a.Ev || !a.gvec || (STRICT && !a.Ev_lo))))) return MLSTM_EINVAL;
+    const size_t lds = Cfg::LDS_BYTES + (a.chunk_len > 0 ? Cfg::EXTRA_CHUNK_BYTES : 0) + (size_t)a.NG * sizeof(float);
+    if (lds > 160 * 1024) return MLSTM_ESHAPE;
+    hipLaunchKernelGGL(kern, dim3(a.BH * a.NG), dim3(256), lds, st, a);
     return (int)hipGetLastError();
 }
 

@@ -61,6 +61,7 @@ struct RowArgs {
     float* rowinter;      //   [BH,S] out: q_i . dQ_i of the state part = the row sums of dD over the keys before the chunk
     const void* Cst;      // [BH][n_states][D][D] matrix states in the element type of X, rows in contraction order:
                           // key-major for the forward, value-major (ChunkArgs::CstT) for the dQ pass
+    const void* Cst_lo;   // split mode: the states' low-order terms, same layout (the state enters its product as Cst + Cst_lo)
     const float* Nst;     // [BH][n_states][D] vector states
     const float* alpha2;
     const float* beta2;
@@ -94,6 +95,7 @@ struct RowArgs {
 int launch_row_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);
 // eight waves (producer / consumer pairs per SIMD); 16-bit types and D in {128, 256} only
 int launch_row8_kernel(int mode, int dtype, int D, const RowArgs& a, hipStream_t st);
+// (the four-wave kernel serves every other case: fp32, D = 64, split mode -- in chunks too -- and the test switch)
 inline int launch_row_best(int mode, int dtype, int D, const RowArgs& a, hipStream_t st) {
     if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic && !a.precise) {
         int rc = launch_row8_kernel(mode, dtype, D, a, st);
@@ -118,6 +120,7 @@ struct ColArgs {
     int chunk_len;
     int n_states;
     const void* Ev;          // [BH][n_states][D][D] reverse states, value-major (ChunkArgs::CstT of the reverse pass)
+    const void* Ev_lo;       // split mode: their low-order terms
     const float* gvec;       // [BH][n_states][D]
     int precise;             // split mode (see RowArgs): G and W enter phase B as hi + lo
     Lay la, lb;              // layouts of Q, K, V, dK, dV (la) and of dH (lb)
@@ -169,11 +172,18 @@ struct ChunkArgs {
     const float* inv_n;
     const float* db;
     Lay lk, lv;           // layouts of K and V
+    // Split mode: the weighted V rows enter the chunk sums as two terms (hi + lo, two MFMAs per fragment) and every state
+    // is written as two terms as well: Cst_lo / CstT_lo receive state - (state rounded to the element type), rounded.
+    int precise;
+    void* Cst_lo;
+    void* CstT_lo;
 };
 int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st);
 
-// anchor[bh][c] = <A_c, B_c> + va_c . vb_c over two sets of states in the same layout
-int launch_anchor(int dtype, int D, const void* A, const void* B, const float* va, const float* vb, float* anchor, int BH, int NCS, hipStream_t st);
+// anchor[bh][c] = <A_c, B_c> + va_c . vb_c over two sets of states in the same layout; A_lo, B_lo (both or neither):
+// their low-order terms (split mode)
+int launch_anchor(int dtype, int D, const void* A, const void* B, const void* A_lo, const void* B_lo, const float* va, const float* vb,
+                  float* anchor, int BH, int NCS, hipStream_t st);
 
 // Backward of the output gate h_out = silu(o) * h, element-wise over n elements (n a multiple of 8):
 //   dh = dh_out * silu(o)   (the upstream gradient of the ungated form),   d_o = dh_out * h * silu'(o).

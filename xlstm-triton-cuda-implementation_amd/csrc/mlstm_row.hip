@@ -15,6 +15,14 @@
 //
 // Memory pipeline: the two 64-key tiles of step j+1 are copied global->LDS by direct loads (no registers) into
 // the other of two LDS stages while step j is consumed; one barrier per step.  Tiles are XOR-swizzled.
+//
+// Long sequences in chunks (RowArgs::chunk_len): a row tile walks the key tiles of its own chunk only; what lies before
+// the chunk enters through the state at the end of the previous chunk (mlstm_chunk.hip), D/64 tiles of 64 state rows
+// that pass through the same LDS stages ahead of the key tiles and are contracted with the rows' own X fragments:
+//   forward  H^T += C~^T-tiles x Q^T, then the rows' decay exp(A_e - A_i), and b += decay (q_i . n~);
+//   dQ pass  dQ^T += C~-tiles (value-major) x dH^T, then decay / n_i, the rank-one term decay db_i n~, and the row sums
+//            q_i . dQ_i of dD over the keys before the chunk.
+// In split mode the state comes as two terms, hi + lo (one tile each per stage), and takes two MFMAs per fragment.
 #include <mutex>
 #include <type_traits>
 #include "mlstm_device.h"
@@ -44,7 +52,7 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
-    const int S = a.S, NG = a.NG;
+    int S = a.S, NG = a.NG;
     const int nQT = (S + ROW_BQ - 1) / ROW_BQ;
     int bh, qt;
     {
@@ -61,12 +69,23 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
             qt = nQT - 1 - bid / a.BH;
         }
     }
+    size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN, goff = (size_t)bh * NG;
+    // the caller's tensors: q, k, v, dq in layout la, h, dh, o in lb (element offset of the head, elements per position)
+    const size_t rsA = (size_t)a.la.ss, rsB = (size_t)a.lb.ss, rsH = (size_t)a.lh.ss;
+    size_t offA = a.la.head(bh), offB = a.lb.head(bh), offH = a.lh.head(bh);
+    // In chunks the workgroup's rows lie in chunk `chunk`, and everything below addresses positions relative to the chunk's
+    // first one: the sequence "starts" there (offsets move forward; S, NG and the row tile index shrink).
+    int chunk = 0;
+    if (a.chunk_len > 0) {
+        chunk = (qt * ROW_BQ) / a.chunk_len;
+        const int p0 = chunk * a.chunk_len;
+        hoff += p0; poff += p0; goff += p0 / GRAN;
+        offA += (size_t)p0 * rsA; offB += (size_t)p0 * rsB; offH += (size_t)p0 * rsH;
+        S -= p0; NG -= p0 / GRAN; qt -= p0 / ROW_BQ;
+    }
     const int q0 = qt * ROW_BQ, r0 = q0 + 32 * wave;
     const int row = r0 + c32, rowc = row < S ? row : S - 1;
     const bool wave_active = r0 < S;
-    const size_t hoff = (size_t)bh * S, poff = (size_t)bh * NG * GRAN;
-    // the caller's tensors: q, k, v, dq in layout la, h, dh, o in lb (element offset of the head, elements per position)
-    const size_t rsA = (size_t)a.la.ss, rsB = (size_t)a.lb.ss, offA = a.la.head(bh), offB = a.lb.head(bh);
     const size_t rsX = MODE == MODE_FWD ? rsA : rsB, offX = MODE == MODE_FWD ? offA : offB;
     const size_t rsO = MODE == MODE_FWD ? rsB : rsA, offO = MODE == MODE_FWD ? offB : offA;
     const T* X = reinterpret_cast<const T*>(a.X) + offX;
@@ -80,13 +99,13 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
     // granule bases of this head in LDS: a global load inside the main loop would have to be waited for with
     // vmcnt(0), which would also wait for the tile copies in flight
     double* const sG = reinterpret_cast<double*>(smem + Cfg::STAGES_BYTES);
-    for (int g = tid; g < NG; g += 256) sG[g] = a.G2[(size_t)bh * NG + g];
+    for (int g = tid; g < NG; g += 256) sG[g] = a.G2[goff + g];
     float crow_base = -0.5f * __log2f((float)D) - a.beta2[poff + rowc];
     float inv_n = 0.f, dbv = 0.f;
     if constexpr (MODE == MODE_DQ) {
         const T* hlo = nullptr;
         if constexpr (STRICT) { if (a.Hin_lo) hlo = reinterpret_cast<const T*>(a.Hin_lo) + (hoff + rowc) * D; }
-        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + a.lh.head(bh) + (size_t)rowc * (size_t)a.lh.ss, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv, hlo);
+        row_stats<T, NS>(xf, reinterpret_cast<const T*>(a.Hin) + offH + (size_t)rowc * rsH, h, a.Bin[hoff + rowc], a.M[hoff + rowc], inv_n, dbv, hlo);
         if (row < S && h == 0) { a.inv_n[poff + row] = inv_n; a.db[poff + row] = dbv; }
     }
 #pragma unroll
@@ -114,7 +133,7 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
 #define ST_AL(st) (reinterpret_cast<float*>(ST_Y2(st) + Cfg::TILE_ELEMS))
     const float* const alpha_head = a.alpha2 + poff;
     const float* const ek_head = a.ek2 + poff;
-    const float* const amax_head = a.amax2 + (size_t)bh * NG * 2;
+    const float* const amax_head = a.amax2 + goff * 2;
     TileDma<T, D, GRAN, 256> tdma;
     tdma.init(tid);
     const auto ra = tdma.rows(tid, (unsigned)(rsA * sizeof(T)));
@@ -314,7 +333,94 @@ __global__ __launch_bounds__(256, 1) void row_kernel(RowArgs a) {
 
     __syncthreads();  // sG visible; every plain global load above has been waited for (pin)
     const double GI = sG[(wave_active ? r0 : S - 1) / GRAN];
-    ROW_DMA(0, 0);
+    if (chunk > 0) {
+        // ---- what lies before the chunk: the state at the end of the previous chunk, as D/64 tiles of 64 rows in the order
+        // in which this product contracts them (mlstm_chunk.hip), hi tile in a stage's Y1 slot and, in split mode, the lo
+        // tile in its Y2 slot.  The last state tile sits in stage 1, so that key tile 0 can follow into stage 0 under it.
+        constexpr int NTL = D / GRAN, NGRP = GRAN / KW;
+        const size_t sbase = ((size_t)bh * a.n_states + chunk - 1) * D * D;
+        const T* const Cs = reinterpret_cast<const T*>(a.Cst) + sbase;
+        const T* const Cl = STRICT ? reinterpret_cast<const T*>(a.Cst_lo) + sbase : nullptr;
+        auto issue_state = [&](int tau) {
+            const int stg = (tau + (NTL & 1)) & 1;
+            tdma.issue(ST_Y1(stg), Cs + (size_t)GRAN * tau * D);
+            if constexpr (STRICT) tdma.issue(ST_Y2(stg), Cl + (size_t)GRAN * tau * D);
+        };
+        issue_state(0);
+        // the rows' decay since the end of the previous chunk: requested now, used behind the tiles
+        const float dec = fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc] + (float)(a.G2[goff + rowc / GRAN] - a.G2[goff - 1]));
+#pragma unroll
+        for (int tau = 0; tau < NTL; tau++) {
+            const int stg = (tau + (NTL & 1)) & 1;
+            dma_wait();
+            __syncthreads();   // tile tau has landed; the other stage is free
+            if (tau + 1 < NTL) issue_state(tau + 1);
+            else ROW_DMA(0, 0);
+            const T* th = ST_Y1(stg);
+            const T* tl = ST_Y2(stg);
+            auto rd = [&](const T* tile, int g, int d) {
+                if constexpr (FAST_TR) return vrd.read(tile, KW * g, d);
+                else return swz_frag_transposed<T, D>(tile, KW * g, 32 * d, lane);
+            };
+            frag vf[2][NDB];
+#pragma unroll
+            for (int d = 0; d < NDB; d++) vf[0][d] = rd(th, 0, d);
+#pragma unroll
+            for (int g = 0; g < NGRP; g++) {
+                frag vl[STRICT ? NDB : 1];
+#pragma unroll
+                for (int d = 0; d < NDB; d++) {
+                    if constexpr (STRICT) vl[d] = rd(tl, g, d);
+                    if (g + 1 < NGRP) vf[(g + 1) & 1][d] = rd(th, g + 1, d);
+                    R::mma(oacc[d], vf[g & 1][d], xf[NGRP * tau + g]);
+                }
+                if constexpr (STRICT) {
+#pragma unroll
+                    for (int d = 0; d < NDB; d++) R::mma(oacc[d], vl[d], xf[NGRP * tau + g]);
+                }
+            }
+        }
+        const float* nst = a.Nst + ((size_t)bh * a.n_states + chunk - 1) * D;
+        if constexpr (MODE == MODE_FWD) {
+            // row sums: decay_i (q_i . n~); the lane's half of the row (the halves meet in the epilogue)
+            float part = 0.f;
+#pragma unroll
+            for (int s2 = 0; s2 < NS; s2++)
+#pragma unroll
+                for (int e = 0; e < R::EPL; e++) part += to_f32(xf[s2][e]) * nst[KW * s2 + R::EPL * h + e];
+            bsum += dec * part;
+#pragma unroll
+            for (int d = 0; d < NDB; d++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[d][r] *= dec;
+        } else {
+            const float decn = dec * inv_n, rank1 = dec * dbv;
+            const T* qrow = reinterpret_cast<const T*>(a.Qrow) + offA + (size_t)rowc * rsA;
+            float rp = 0.f;
+#pragma unroll
+            for (int d = 0; d < NDB; d++)
+#pragma unroll
+                for (int a4 = 0; a4 < 4; a4++) {
+                    const int col = 32 * d + 8 * a4 + 4 * h;
+                    const f32x4 nv = *reinterpret_cast<const f32x4*>(nst + col);
+                    const f32x4 qv = __builtin_convertvector(*reinterpret_cast<const typename R::vec4*>(qrow + col), f32x4);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const float v = oacc[d][4 * a4 + c] * decn + rank1 * nv[c];
+                        oacc[d][4 * a4 + c] = v;
+                        rp += v * qv[c];
+                    }
+                }
+            // row sums of dD over the keys before the chunk: q_i . dQ_i of what the accumulators hold now
+            rp = sum_halves(rp);
+            if (row < S && h == 0) a.rowinter[hoff + row] = rp;
+        }
+    } else {
+        if constexpr (MODE == MODE_DQ) {
+            if (a.chunk_len > 0 && row < S && h == 0) a.rowinter[hoff + row] = 0.f;
+        }
+        ROW_DMA(0, 0);
+    }
     // Tiles strictly below this wave's rows take the mask-free path; the last one or two tiles of the workgroup are
     // diagonal, or entirely above the diagonal, for this wave.  Two loops with one code path each keep the output
     // accumulators in place (a two-way branch inside one loop makes the register allocator copy them every step).
