@@ -367,6 +367,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
+    ap.add_argument("--column-kernel", type=int, default=0, choices=[0, 1, 2, 3],
+                    help="measurement aid: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (torch), twice, before the steps: under rocprofv3 --pmc its "
                          "FETCH_SIZE / WRITE_SIZE readings calibrate the counters' unit")
@@ -380,6 +382,7 @@ def main():
 
     from _mlstm_pkg import submodule
     ffi = submodule("_ffi")
+    ffi.set_column_kernel(args.column_kernel)
     if args.calibrate_copy:
         # 1 GiB, copied twice: four times the chip's 256 MB last-level cache, so the second copy's source comes from HBM
         # (a source that still sits in that cache reads as almost no FETCH_SIZE at all)

@@ -312,6 +312,13 @@ int mlstm_force_generic_kernels(int on);
  * Workspace sizes depend on it: query mlstm_workspace_bytes after changing it.
  */
 int mlstm_set_chunk_length(int length);
+/*
+ * Measurement and test aid: which column kernel (dK, dV, dI) serves the 16-bit types at D = 128 and 256.
+ * 0 = the library's choice, 1 = col16_kernel (G / W through LDS, 16x16 MFMA chains), 2 = cold_kernel (G / W stay in
+ * registers; the only one of the two with a split mode), 3 = the generic four-wave col_kernel.  Process-wide; returns 0,
+ * or MLSTM_EINVAL.  No counterpart in the reference.
+ */
+int mlstm_set_column_kernel(int variant);
 /* The chunk length the entry points use for this shape under the current setting, 0 = the sequence is not cut
  * (measurement aid: the work a chunked kernel executes depends on it). */
 int mlstm_chunk_length_for(int S, int D, int dtype);

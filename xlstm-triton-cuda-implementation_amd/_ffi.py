@@ -101,6 +101,8 @@ def lib():
         L.mlstm_kernel_error.argtypes = []
         L.mlstm_init.restype = ci
         L.mlstm_init.argtypes = []
+        L.mlstm_set_column_kernel.restype = ci
+        L.mlstm_set_column_kernel.argtypes = [ci]
         L.mlstm_set_spin_limit.restype = ci
         L.mlstm_set_spin_limit.argtypes = [ci]
         L.mlstm_force_generic_kernels.restype = ci
@@ -117,7 +119,7 @@ def exported_symbols():
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
-            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init"]
+            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init", "mlstm_set_column_kernel"]
 
 
 KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
@@ -127,6 +129,11 @@ KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state
 def force_generic_kernels(on):
     """Test aid: route every shape through the generic four-wave kernels; returns the previous setting."""
     return bool(lib().mlstm_force_generic_kernels(1 if on else 0))
+
+
+def set_column_kernel(variant):
+    """Measurement and test aid: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel."""
+    check_rc(lib().mlstm_set_column_kernel(int(variant)), "mlstm_set_column_kernel")
 
 
 def set_chunk_length(length):

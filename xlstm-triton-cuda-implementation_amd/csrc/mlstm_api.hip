@@ -9,6 +9,7 @@ using namespace mlstm;
 
 namespace mlstm {
 bool g_force_generic = false;  // see mlstm_force_generic_kernels
+int g_col_variant = 0;         // see mlstm_set_column_kernel
 }
 
 namespace {
@@ -404,6 +405,12 @@ int mlstm_force_generic_kernels(int on) {
     const int before = mlstm::g_force_generic ? 1 : 0;
     mlstm::g_force_generic = on != 0;
     return before;
+}
+
+int mlstm_set_column_kernel(int variant) {
+    if (variant < 0 || variant > 3) return MLSTM_EINVAL;
+    mlstm::g_col_variant = variant;
+    return 0;
 }
 
 int mlstm_chunk_length_for(int S, int D, int dtype) {

@@ -129,10 +129,18 @@ int launch_col_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
 // phase A as 16x16x32 products on two query halves, the element-wise part of the first between the MFMAs of the second;
 // 16-bit types at D = 128 and 256 only
 int launch_col16_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
+// weights kept in registers between the two phases (no G / W tiles in LDS); 16-bit types at D = 128 and 256, split mode included
+int launch_cold_kernel(int dtype, int D, const ColArgs& a, hipStream_t st);
+extern int g_col_variant;   // see mlstm_set_column_kernel: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel
 inline int launch_col_best(int dtype, int D, const ColArgs& a, hipStream_t st) {
-    if (dtype != MLSTM_F32 && (D == 128 || D == 256) && !g_force_generic && !a.precise) {
-        int rc = launch_col16_kernel(dtype, D, a, st);
-        if (rc != MLSTM_ESHAPE) return rc;  // extremely long sequences do not fit its LDS budget
+    const bool half_big = dtype != MLSTM_F32 && (D == 128 || D == 256);
+    int variant = g_force_generic ? 3 : g_col_variant;
+    if (!half_big || variant < 0 || variant > 3) variant = 3;
+    if (variant == 0) variant = a.precise ? 2 : 1;
+    if (variant == 1 && a.precise) variant = 2;   // (col16_kernel has no split mode)
+    if (variant == 1 || variant == 2) {
+        int rc = variant == 1 ? launch_col16_kernel(dtype, D, a, st) : launch_cold_kernel(dtype, D, a, st);
+        if (rc != MLSTM_ESHAPE) return rc;  // extremely long sequences do not fit their LDS budget
     }
     return launch_col_kernel(dtype, D, a, st);
 }
