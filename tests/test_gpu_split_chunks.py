@@ -128,3 +128,39 @@ def test_saved_buffer_of_another_setting_is_reported():
     with chunk_length(128):
         mm.mlstm_backward_saved_hip(*args, h, m, b, saved)
     assert L.mlstm_kernel_error() == 0
+
+
+class column_kernel:
+    def __init__(self, variant):
+        self.variant = variant
+
+    def __enter__(self):
+        ffi.set_column_kernel(self.variant)
+
+    def __exit__(self, *exc):
+        ffi.set_column_kernel(0)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("variant", [1, 2, 3])
+@pytest.mark.parametrize("B,NH,S,D,L", [(1, 2, 97, 128, -1), (1, 2, 330, 256, -1), (1, 2, 520, 256, 128), (1, 3, 1000, 128, 256), (2, 8, 1536, 256, 0)])
+def test_every_column_kernel_against_the_oracle(dt, variant, B, NH, S, D, L):
+    """The three column kernels (dK, dV, dI; with the dF pass behind them) that serve the 16-bit types at D = 128 and 256
+    -- col16_kernel, cold_kernel (the default) and the generic col_kernel -- on the same inputs: ragged lengths, with and
+    without chunks, a multiple of eight heads (the workgroup order by XCD); each under the rule of the default kernels,
+    cold_kernel and col_kernel in split mode at the literal bound as well."""
+    dtype = DT[dt]
+    q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=S + D + variant, f_mean=2.0)
+    args = dev(dh, q, k, v, f, i)
+    heads = [(0, 0), (B - 1, NH - 1)]
+    with chunk_length(L):
+        Lc = int(ffi.lib().mlstm_chunk_length_for(S, D, ffi.dtype_code(dtype)))
+        for precise in ([False] if variant == 1 else [False, True]):
+            with column_kernel(variant):
+                h, m, b, saved = mm.mlstm_forward_save_hip(*args[1:], precise=precise)
+                got = mm.mlstm_backward_saved_hip(*args, h, m, b, saved, precise=precise)
+            for (bi, hi) in heads:
+                one = [x[bi:bi + 1, hi:hi + 1] for x in (q, k, v, f, i, dh)]
+                assert_matches_oracle(dtype, *one, grads=[g_[bi:bi + 1, hi:hi + 1] for g_ in got], chunk_len=Lc, precise=precise,
+                                      tag=f"kernel {variant} precise={precise} [{bi},{hi}] ")
+    assert ffi.lib().mlstm_kernel_error() == 0

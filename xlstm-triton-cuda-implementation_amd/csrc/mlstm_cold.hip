@@ -33,7 +33,7 @@ struct ColdCfg {
     static constexpr size_t QT_BYTES = (size_t)CD_QT * D * sizeof(T);                  // a 32-row tile of Q or dH
     static constexpr size_t STAGES_BYTES = 4 * QT_BYTES;                               // two stages of (Q, dH); the state tiles before them
     static constexpr size_t ROW_BYTES = 2 * 3 * GRAN * sizeof(float);                  // per stage: beta, 1/n, db (64 floats copied, 32 used)
-    static constexpr size_t MISC_BYTES = (2 * 4 * CD_QT + 64) * sizeof(float);         // row sums [2 parities][4 key blocks][32], 64 sink words
+    static constexpr size_t MISC_BYTES = (2 * 4 * CD_QT + 64 + D) * sizeof(float);     // row sums [2 parities][4 key blocks][32], 64 sink words, the vector state
     static constexpr size_t LDS_BYTES = V_BYTES + STAGES_BYTES + ROW_BYTES + MISC_BYTES;   // plus one float per 64-position granule
 };
 
@@ -80,9 +80,23 @@ template <> struct MmaV<_Float16> {
 };
 __device__ __forceinline__ void settle(f32x16& c0, f32x16& c1) { asm volatile("s_nop 15\n\ts_nop 15" : "+v"(c0), "+v"(c1)); }
 
+// Profiling builds (-DMLSTM_COLD_PROF): waves 0 and 3 add up the shader-clock cycles they spend in each part of the
+// kernel and leave the sums, as floats, in the first two rows of the workgroup's dK tile (the results are then wrong, the
+// timing is what the build is for).  s_memtime is only trustworthy with one wave per SIMD, which this kernel has.
+#ifdef MLSTM_COLD_PROF
+#define CP_DECL float prof_[12] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; long long last_ = (long long)__builtin_amdgcn_s_memtime()
+#define CP_STAMP(k) do { const long long now_ = (long long)__builtin_amdgcn_s_memtime(); prof_[k] += (float)(now_ - last_); last_ = now_; } while (0)
+#define CP_COUNT(k) do { prof_[k] += 1.f; } while (0)
+#else
+#define CP_DECL do {} while (0)
+#define CP_STAMP(k) do {} while (0)
+#define CP_COUNT(k) do {} while (0)
+#endif
+
 template <typename T, int D, bool STRICT, bool DENSE>
 __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)  // the body uses device-only builtins; the host pass only needs the stub
+    CP_DECL;
     using R = Tr<T>;
     using Cfg = ColdCfg<T, D>;
     using Z = Swz<T, D>;
@@ -98,7 +112,8 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
 #define ST_DH(st) (reinterpret_cast<T*>(stg + (size_t)(2 * (st) + 1) * Cfg::QT_BYTES))
 #define ST_ROW(st) (reinterpret_cast<float*>(tail) + (st) * 3 * GRAN)
     float* const rowtmp = reinterpret_cast<float*>(tail + Cfg::ROW_BYTES);   // [2][4][32]
-    float* const sG = rowtmp + 2 * 4 * CD_QT + 64;   // (behind the sink words) granule bases minus that of the tile's first granule
+    float* const gvl = rowtmp + 2 * 4 * CD_QT + 64;   // (behind the sink words) the chunk's vector state g
+    float* const sG = gvl + D;                         // granule bases minus that of the tile's first granule
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
     const int kb = wave;
@@ -209,6 +224,7 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
     SwzRowReaderX<T, D> rrd;
     rrd.init(lane);
 
+    if (has_state && tid < D) gvl[tid] = a.gvec[((size_t)bh * a.n_states + chunk) * D + tid];
     if (tid < NG) sG[tid] = (float)(g_first - gbase);
     for (int g = tid + 256; g < NG; g += 256) sG[g] = (float)(a.G2[goff + g] - gbase);
     const float gcorr = (float)(gbase - gkey);   // granule base of the tile's first granule minus that of the wave's keys
@@ -216,18 +232,43 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
     for (int s = 0; s < NS; s++) pin(kf[s]);
     dma_wait();
     __syncthreads();   // V of the keys and the first state piece (or the first query tile) have landed; sG is visible
+    CP_STAMP(0);
 
     // ---- state phase (sequences in chunks): E is stored value-major (row = value index, rows in the contraction order of
     // the transposing reads).  Per piece of SROWS rows: dK contracts over the piece's rows (values) with V out of LDS; dV
     // is owed by the piece's own rows (SROWS / 32 blocks of output columns), contracted over the whole key index with the
     // K fragments in registers.
     float colacc = 0.f;   // the lane's share of the column sum of dD of its key
+    // Scaling by the keys' weights w_j.  bf16 (END_SCALE): instead of multiplying all 2 D accumulators of a lane by w_j
+    // behind the state phase (some two thousand instructions: every accumulator through the vector registers and back), the
+    // query loop divides ITS contributions by s_j = w_j (the weights' exponent subtracts log2 s_j, exact in fp32, and bf16 has
+    // fp32's range), and the epilogue multiplies the sums by s_j once, where it touches every element anyway, and adds
+    // w_j g there.  A key whose weight is below 2^-40 drops the state part instead (its operands are zeroed) and uses
+    // s_j = 1: what it loses is below 2^-40 of the state product.  fp16 cannot hold G / s_j and scales the accumulators.
+    constexpr bool END_SCALE = std::is_same<T, __bf16>::value;
+    float scale_s = 1.f, log2_s = 0.f, wkg = 0.f;   // s_j, its log2, and w_j for the epilogue's w_j g (0 without a state)
     if (has_state) {
         const float wk = fast_exp2(al - bend + (float)(Gend - gkey));
+        const bool use = !END_SCALE || wk > 0x1p-40f;
+        if constexpr (END_SCALE) {
+            if (use) { scale_s = wk; log2_s = al - bend + (float)(Gend - gkey); }
+            wkg = wk;
+        }
         // the stored place of the lane's own row c32 inside a 32-row block (rows are kept in the contraction order of the
         // transposing reads: the two middle groups of four of every 16 swap places), as a byte offset with the column half
         const int own_row = (c32 & ~15) | ((c32 & 3) | ((c32 & 4) << 1) | ((c32 & 8) >> 1));
         const int own_off = Z::off(own_row, R::EPL * h);
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        auto masked = [&](frag f) {   // (END_SCALE: a key that drops the state part multiplies with zeros)
+            if constexpr (END_SCALE) {
+                i32x4 bits = __builtin_bit_cast(i32x4, f);
+#pragma unroll
+                for (int e = 0; e < 4; e++) bits[e] = use ? bits[e] : 0;
+                return __builtin_bit_cast(frag, bits);
+            } else {
+                return f;
+            }
+        };
 #pragma unroll
         for (int p = 0; p < NPIECE; p++) {
             if (p + 1 < NPIECE) state_issue(p + 1);   // (into the slots piece p - 1 left behind the last barrier)
@@ -235,7 +276,7 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
             const T* tl = piece_lo(p);
 #pragma unroll
             for (int t16 = 0; t16 < SROWS / KW; t16++) {
-                const frag vB = rrd.read(Vt, kb, (SROWS / KW) * p + t16);
+                const frag vB = masked(rrd.read(Vt, kb, (SROWS / KW) * p + t16));
 #pragma unroll
                 for (int x = 0; x < NXD; x++) {
                     R::mma(dkacc[x], trd.read(th, KW * t16, x), vB);
@@ -251,37 +292,53 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
 #pragma unroll
                 for (int t = 0; t < NS; t++) {
                     const int o = (own_off ^ ((t % 8) << 5)) + (t / 8) * 256;
-                    R::mma(dvacc[(SROWS / 32) * p + xx], *reinterpret_cast<const frag*>(eh + o), kf[t]);
-                    if constexpr (STRICT) R::mma(dvacc[(SROWS / 32) * p + xx], *reinterpret_cast<const frag*>(el + o), kf[t]);
+                    const frag kB = masked(kf[t]);
+                    R::mma(dvacc[(SROWS / 32) * p + xx], *reinterpret_cast<const frag*>(eh + o), kB);
+                    if constexpr (STRICT) R::mma(dvacc[(SROWS / 32) * p + xx], *reinterpret_cast<const frag*>(el + o), kB);
                     if (t % 4 == 3) __builtin_amdgcn_sched_barrier(0);
                 }
             }
             dma_wait();
             __syncthreads();   // every wave is done with piece p, and piece p + 1 has landed
         }
+        CP_STAMP(1);
         COLD_DMA(it0, 0);   // the first query tile follows the state into stage 0
-        // the keys' weights, the vector state and k_j . dK_j, which goes into the column sums
-        const float* gv = a.gvec + ((size_t)bh * a.n_states + chunk) * D;
-        const T* krow = K + (size_t)keyc * rsA;
+        // k_j . (E v_j + g) w_j, the column sums of dD over the queries behind the chunk (and, for fp16, the scaling itself).
+        // The K values a lane needs (its accumulators' rows 8 a4 + 4 h + c of every block) are in the K fragments of the two
+        // lanes of its key (which hold columns 16 s + 8 h + 0..7): one v_permlane32_swap per register pair sorts them out.
         float cp = 0.f;
 #pragma unroll
-        for (int x = 0; x < NXD; x++) {
+        for (int s = 0; s < NS; s++) {
+            const int x = s >> 1, a4a = 2 * (s & 1);
+            const i32x4 w = __builtin_bit_cast(i32x4, kf[s]);
+            const auto r0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+            const auto r1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+            typedef int i32x2 __attribute__((ext_vector_type(2)));
+            // first results: columns 16 s + 4 h + c (own low half for h = 0, the partner's high half for h = 1); second
+            // results: columns 16 s + 8 + 4 h + c
+            const f32x4 ka = __builtin_convertvector(__builtin_bit_cast(typename R::vec4, i32x2{(int)r0[0], (int)r1[0]}), f32x4);
+            const f32x4 kc = __builtin_convertvector(__builtin_bit_cast(typename R::vec4, i32x2{(int)r0[1], (int)r1[1]}), f32x4);
 #pragma unroll
-            for (int a4 = 0; a4 < 4; a4++) {
-                const int d = 32 * x + 8 * a4 + 4 * h;
-                const f32x4 g4v = *reinterpret_cast<const f32x4*>(gv + d);
-                const f32x4 kv = __builtin_convertvector(*reinterpret_cast<const typename R::vec4*>(krow + d), f32x4);
+            for (int u = 0; u < 2; u++) {
+                const int a4 = a4a + u;
+                const f32x4 g4v = *reinterpret_cast<const f32x4*>(gvl + 32 * x + 8 * a4 + 4 * h);
 #pragma unroll
                 for (int c = 0; c < 4; c++) {
-                    const float dkv = (dkacc[x][4 * a4 + c] + g4v[c]) * wk;
-                    dkacc[x][4 * a4 + c] = dkv;
-                    dvacc[x][4 * a4 + c] *= wk;
-                    cp += dkv * kv[c];
+                    const float kval = u ? kc[c] : ka[c];
+                    if constexpr (END_SCALE) {
+                        cp += (dkacc[x][4 * a4 + c] + g4v[c]) * kval;
+                    } else {
+                        const float dkv = (dkacc[x][4 * a4 + c] + g4v[c]) * wk;
+                        dkacc[x][4 * a4 + c] = dkv;
+                        dvacc[x][4 * a4 + c] *= wk;
+                        cp += dkv * kval;
+                    }
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);   // (one block of the accumulators at a time through the vector registers)
+            if (s % 2 == 1) __builtin_amdgcn_sched_barrier(0);   // (one block of the accumulators at a time through the vector registers)
         }
-        colacc = cp;   // (the far column sum starts the lane's column accumulator: the two halves of the wave meet in the epilogue)
+        colacc = END_SCALE ? cp * wk : cp;   // (starts the lane's column accumulator: the two halves of the wave meet in the epilogue)
+        CP_STAMP(2);
     }
     const float log2scale = -0.5f * __log2f((float)D);
 
@@ -299,6 +356,8 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
         const int stage = (it - it0) & 1, stn = stage ^ 1;
         dma_wait();
         __syncthreads();   // tile `it` has landed and every wave is past phase B of the previous step
+        CP_STAMP(3);
+        CP_COUNT(8);
         if constexpr (SPREAD) {
             rvdma.issue(ST_ROW(stn), it + 1);
         } else {
@@ -352,26 +411,35 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (D == 256) settle(wacc, gacc);
+            CP_STAMP(4);
+            CP_COUNT(9);
             // ---- element-wise part and phase B, by halves of the tile's queries: registers 8t .. 8t+7 of a block are the 16
             // queries of contraction step t of phase B, so the second half's element-wise work, and all the lane reductions
             // of the row sums, are placed between the MFMAs of phase B.  Everything is branch-free: a masked element (key
             // behind the query, or a query past the end) gets the exponent -inf.
-            const float argbase = al + (sG[it >> 1] + gcorr + log2scale);
+            const float argbase = al + (sG[it >> 1] + gcorr + log2scale) - log2_s;   // (weights over s_j: see END_SCALE)
             const unsigned span = (unsigned)(S - key);    // query q takes part iff 0 <= q - key < S - key (unsigned compare)
             const int dq0 = qi0 + 4 * h - key;            // q - key of register r: dq0 + 8 (r / 4) + r % 4
             float dd[16];
+            f32x4 beta4[2], inv4[2], db4[2];   // the scalars of the half's eight queries (two groups of four registers)
+            auto ew_scalars = [&](int t) {
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const int ql = 8 * (2 * t + u) + 4 * h;
+                    beta4[u] = *reinterpret_cast<const f32x4*>(srow + ql);
+                    inv4[u] = *reinterpret_cast<const f32x4*>(srow + GRAN + ql);
+                    db4[u] = *reinterpret_cast<const f32x4*>(srow + 2 * GRAN + ql);
+                }
+            };
             auto ew_one = [&](int r) {
-                const int ql = 8 * (r >> 2) + 4 * h + (r & 3);
-                float beta = srow[ql];
-                const float inv = srow[GRAN + ql], db = srow[2 * GRAN + ql];
-                asm volatile("" : "+v"(beta));   // (keeps the read out of the select below, which would otherwise become a branch)
-                const bool live = (unsigned)(dq0 + 8 * (r >> 2) + (r & 3)) < span;
-                const float e = fast_exp2(live ? argbase - beta : -INFINITY);
+                const int u = (r >> 2) & 1, c = r & 3;
+                const bool live = (unsigned)(dq0 + 8 * (r >> 2) + c) < span;
+                const float e = fast_exp2(live ? argbase - beta4[u][c] : -INFINITY);
                 const float ct = wacc[r] * e;
-                const float dct = gacc[r] * inv + db;
-                dd[r] = ct * dct;
+                const float dct = gacc[r] * inv4[u][c] + db4[u][c];
+                dd[r] = END_SCALE ? (ct * scale_s) * dct : ct * dct;
                 gacc[r] = dct * e;
-                wacc[r] = ct * inv;
+                wacc[r] = ct * inv4[u][c];
                 colacc += dd[r];
             };
             // lane 15 of a 16-lane row holds the row's total: rows 0 / 2 (h = 0 / 1) carry register 2p, rows 1 / 3 register
@@ -383,11 +451,14 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
                 float* dst = (lane & 15) == 15 ? rt + (8 * (r >> 2) + 4 * h + (r & 3)) : sink;
                 *dst = tot;
             };
+            ew_scalars(0);
 #pragma unroll
             for (int r = 0; r < 8; r++) ew_one(r);
+            ew_scalars(1);   // (for the second half, whose work rides on phase B below)
             float rs[8];
 #pragma unroll
             for (int p = 0; p < 4; p++) rs[p] = fold_pair(dd[2 * p], dd[2 * p + 1]);
+            CP_STAMP(5);
 #pragma unroll
             for (int t = 0; t < 2; t++) {
                 frag ghi, glo, whi, wlo;
@@ -427,6 +498,7 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
                     for (int p = 4; p < 8; p++) rs[p] = fold_pair(dd[2 * p], dd[2 * p + 1]);
                 }
             }
+            CP_STAMP(6);
         } else {
             if constexpr (SPREAD) { qdma.issue(lq, gq, ra); qdma.issue(ldh, gdh, rb); }
             if (lane < CD_QT) rt[lane] = 0.f;
@@ -464,10 +536,14 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
             for (int x = 0; x < NXD; x++)
 #pragma unroll
                 for (int a4 = 0; a4 < 4; a4++) {
+                    const int d = 32 * x + 8 * a4 + 4 * h;               // first of the four columns
                     f32x4 v;
 #pragma unroll
                     for (int c = 0; c < 4; c++) v[c] = which ? dvacc[x][4 * a4 + c] : dkacc[x][4 * a4 + c];
-                    const int d = 32 * x + 8 * a4 + 4 * h;               // first of the four columns
+                    if constexpr (END_SCALE) {   // the keys' weights: see the state phase
+                        v *= scale_s;
+                        if (!which && has_state) v += *reinterpret_cast<const f32x4*>(gvl + d) * wkg;
+                    }
                     const int chunk16 = (d * (int)sizeof(T)) >> 4, within = (d * (int)sizeof(T)) & 15;
                     *reinterpret_cast<typename R::vec4*>(out + row * ROWB + (((chunk16 ^ (row & 31)) & (CPR - 1)) << 4) + within) = R::cvt4(v);
                 }
@@ -486,6 +562,15 @@ __global__ __launch_bounds__(256, 1) void cold_kernel(ColArgs a) {
             }
         }
     }
+#ifdef MLSTM_COLD_PROF
+    CP_STAMP(7);
+    if ((wave == 0 || wave == 3) && lane < 12 && CD_KEYS * jt + 1 < S) {
+        float v = 0.f;
+#pragma unroll
+        for (int k = 0; k < 12; k++) v = lane == k ? prof_[k] : v;
+        reinterpret_cast<float*>(reinterpret_cast<char*>(a.dK) + (offA + ((size_t)CD_KEYS * jt + (wave == 3)) * rsA) * sizeof(T))[lane] = v;
+    }
+#endif
 #undef ST_Q
 #undef ST_DH
 #undef ST_ROW

@@ -136,7 +136,7 @@ inline int launch_col_best(int dtype, int D, const ColArgs& a, hipStream_t st) {
     const bool half_big = dtype != MLSTM_F32 && (D == 128 || D == 256);
     int variant = g_force_generic ? 3 : g_col_variant;
     if (!half_big || variant < 0 || variant > 3) variant = 3;
-    if (variant == 0) variant = a.precise ? 2 : 1;
+    if (variant == 0) variant = 2;   // (measured faster than col16_kernel at D = 128 and 256, chunked and not)
     if (variant == 1 && a.precise) variant = 2;   // (col16_kernel has no split mode)
     if (variant == 1 || variant == 2) {
         int rc = variant == 1 ? launch_col16_kernel(dtype, D, a, st) : launch_cold_kernel(dtype, D, a, st);
