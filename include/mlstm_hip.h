@@ -72,6 +72,7 @@ typedef struct mlstm_layout {
 #define MLSTM_ESHAPE (-2)      /* head dimension / sequence length not supported by this build */
 #define MLSTM_EWORKSPACE (-3)  /* caller workspace smaller than mlstm_workspace_bytes() */
 #define MLSTM_EKERNEL (-4)     /* a kernel's bounded wait expired (mlstm_kernel_error) */
+#define MLSTM_EBUILD (-6)      /* a kernel with hand-counted memory waits was compiled with register spills: refused */
 #define MLSTM_ESAVED (-5)      /* a backward was given a `saved` buffer written for another shape or setting (mlstm_kernel_error) */
 
 /* operations, for mlstm_workspace_bytes */

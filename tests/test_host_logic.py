@@ -44,3 +44,17 @@ def test_gradient_buffers_of_a_strided_view_keep_its_strides_and_do_not_alias():
     assert g.stride() == fused.stride() and not ffi.overlaps(g)
     g.fill_(1.0)
     assert float(g.sum()) == B * NH * S * D
+
+
+def test_tile_copy_index_arithmetic_stays_inside_the_tiles():
+    """tests/harness/tile_bounds (the kernels' own offset functions, compiled for the host): every block of every tile shape
+    is fetched exactly once, lands where the LDS readers expect it, and no fetch ends beyond the tile's last row -- for the
+    last tile of the last head that is the end of the caller's tensor; the early touch of the dQ pass stays inside its half row."""
+    import os
+    import subprocess
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "harness")
+    exe = os.path.join(here, "tile_bounds")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-C", here, "tile_bounds"])
+    out = subprocess.run([exe], capture_output=True, text=True)
+    assert out.returncode == 0 and "tile_bounds: ok" in out.stdout, out.stdout + out.stderr

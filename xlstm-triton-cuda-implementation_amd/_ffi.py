@@ -16,7 +16,8 @@ _ERRORS = {-1: "invalid argument (null pointer, non-positive size or unknown dty
            -2: "unsupported shape (head dimension / sequence length)",
            -3: "workspace (or saved buffer) too small or of the wrong size",
            -4: "a kernel's bounded wait expired",
-           -5: "a backward was given a saved buffer written for another shape or setting"}
+           -5: "a backward was given a saved buffer written for another shape or setting",
+           -6: "a kernel with hand-counted memory waits was compiled with register spills"}
 
 GATE_FORMS = {"raw": 0, "logsigmoid": 1, "cumsum": 2}   # MLSTM_GATE_RAW / _LOGSIGMOID / _CUMSUM
 

@@ -209,12 +209,12 @@ struct Swz {
     static constexpr int CPR = D / EPC;          // chunks per row
     static constexpr int ROW_BYTES = D * sizeof(T);
     static_assert(CPR >= 8 && (CPR & (CPR - 1)) == 0, "row must be a power-of-two number of chunks, at least 128 bytes");
-    static __device__ __forceinline__ int key(int r) {
+    static __host__ __device__ __forceinline__ int key(int r) {
         if constexpr (CPR >= 16) return ((r & 3) << 2) | ((r >> 2) & 3);
         else return (r >> 1) & 7;
     }
     // byte offset of element column `col` (a multiple of the access width) of row r
-    static __device__ __forceinline__ int off(int r, int col) {
+    static __host__ __device__ __forceinline__ int off(int r, int col) {
         const int c = col / EPC, w = col % EPC;
         return r * ROW_BYTES + (((c ^ key(r))) << 4) + w * (int)sizeof(T);
     }
@@ -290,15 +290,22 @@ struct TileDma {
     static constexpr int GROUP_BYTES = PERIOD * RSTEP * Z::ROW_BYTES;   // global and LDS distance of blocks it and it + PERIOD
     unsigned voff[PERIOD];
     int wave_s;  // wave index as a scalar
+    // Byte offset, from the tile's first row in memory, of the 16 bytes lane `lane` of wave `wave` fetches in its block
+    // `it` (rows `row_bytes` apart); the data lands at byte (it * NW + wave) * 1024 + 16 * lane of the LDS tile.  The
+    // kernels keep lane_source(it) for it < PERIOD only and add (it / PERIOD) * group_bytes(row_bytes) for the others;
+    // a host-side check (tests/harness/tile_bounds.hip) walks every block of every tile shape and asserts that the two
+    // agree, that every 16-byte piece of the tile is fetched exactly once, and that no fetch ends beyond the tile's last row.
+    static __host__ __device__ __forceinline__ unsigned lane_source(int it, int wave, int lane, unsigned row_bytes) {
+        const int p = (it * NW + wave) * 64 + lane;
+        const int r = p / Z::CPR, pc = p % Z::CPR;
+        return (unsigned)r * row_bytes + (unsigned)((pc ^ Z::key(r)) << 4);
+    }
+    static __host__ __device__ __forceinline__ unsigned group_bytes(unsigned row_bytes) { return (unsigned)(PERIOD * RSTEP) * row_bytes; }
     __device__ __forceinline__ void init(int tid) {
         wave_s = __builtin_amdgcn_readfirstlane(tid >> 6);
         const int lane = tid & 63;
 #pragma unroll
-        for (int it = 0; it < PERIOD; it++) {
-            const int p = (it * NW + wave_s) * 64 + lane;
-            const int r = p / Z::CPR, pc = p % Z::CPR;
-            voff[it] = (unsigned)(r * Z::ROW_BYTES + ((pc ^ Z::key(r)) << 4));
-        }
+        for (int it = 0; it < PERIOD; it++) voff[it] = lane_source(it, wave_s, lane, Z::ROW_BYTES);
     }
     // g_tile: first row of the tile (the same for all lanes); tile: LDS destination
     // Blocks [first, last) of this wave only: the kernels spread a tile's copy over the matrix work of the previous
@@ -334,12 +341,8 @@ struct TileDma {
         Rows o;
         const int lane = tid & 63;
 #pragma unroll
-        for (int it = 0; it < PERIOD; it++) {
-            const int p = (it * NW + wave_s) * 64 + lane;
-            const int r = p / Z::CPR, pc = p % Z::CPR;
-            o.voff[it] = (unsigned)r * row_bytes + (unsigned)((pc ^ Z::key(r)) << 4);
-        }
-        o.group_bytes = (unsigned)(PERIOD * RSTEP) * row_bytes;
+        for (int it = 0; it < PERIOD; it++) o.voff[it] = lane_source(it, wave_s, lane, row_bytes);
+        o.group_bytes = group_bytes(row_bytes);
         return o;
     }
     __device__ __forceinline__ void issue_range(T* tile, const T* g_tile_v, int first, int last, const Rows& o) const {
@@ -356,6 +359,13 @@ struct TileDma {
     }
     __device__ __forceinline__ void issue(T* tile, const T* g_tile_v, const Rows& o) const { issue_range(tile, g_tile_v, 0, PER_WAVE, o); }
 };
+
+// Early touch of a row's cache lines by the two lanes (h = 0, 1) that own the row in the eight-wave row kernel: lane h reads
+// one word of line ln + h, ln = 0, 2, ...; a half row of `half_row_bytes` has half_row_bytes / 128 lines and a lane must not
+// go past the last of them (at D = 128 a 16-bit half row is ONE line).  Shared with the host-side bounds check.
+__host__ __device__ constexpr int row8_touch_lines(int half_row_bytes) { return half_row_bytes / 128; }
+__host__ __device__ constexpr bool row8_touch_ok(int ln, int h, int lines) { return ln + h < lines; }
+__host__ __device__ constexpr int row8_touch_offset(int ln, int h) { return 128 * (ln + h); }
 
 // 64 floats (one per key of a tile) by the first wave
 __device__ __forceinline__ void vec64_dma(float* dst, const float* src, int tid) {

@@ -15,6 +15,20 @@ inline hipError_t lds_limit_once(int bytes) {
     static const hipError_t rc = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
     return rc;
 }
+// For kernels whose waits for memory are counted by hand (s_waitcnt vmcnt(n) with n derived from the operations the SOURCE
+// issues): a register spill adds memory operations of the compiler's that the count does not know, and the wait would then
+// let a load pass as landed that has not.  Asked once per process and kernel: the launch is refused (MLSTM_EBUILD) if the
+// compiled kernel uses any scratch memory at all.
+template <auto KERN>
+inline int no_scratch_once() {
+    static const int rc = [] {
+        hipFuncAttributes attr;
+        const hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void*>(KERN));
+        if (e != hipSuccess) return (int)e;
+        return attr.localSizeBytes == 0 ? 0 : MLSTM_EBUILD;
+    }();
+    return rc;
+}
 constexpr int GATE_GRANULE = 64;  // positions per gate granule (== mlstm::GRAN in the device code)
 
 // Where a [B,NH,S,D] (or [B,NH,S]) tensor of the caller's keeps position s of head bh = b * NH + h: at element

@@ -500,13 +500,13 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         int touched[2] = {0, 0};
         if (MODE == R8_DQ && chunk > 0) {
             const char* qb = reinterpret_cast<const char*>(a.Qrow) + (offA + (size_t)dh * (D / 2)) * sizeof(T);
-            constexpr int LINES = (D / 2) * (int)sizeof(T) / 128;   // 128-byte lines of this wave's half of a row
+            constexpr int LINES = row8_touch_lines((D / 2) * (int)sizeof(T));   // 128-byte lines of this wave's half of a row
 #pragma unroll
             for (int r = 0; r < 2; r++) {
 #pragma unroll
                 for (int ln = 0; ln < LINES; ln += 2) {
-                    if (ln + h < LINES)   // (the two lanes of a row take a line each; never past the end of the half row)
-                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * rsA * sizeof(T) + 128 * (ln + h));
+                    if (row8_touch_ok(ln, h, LINES))   // (the two lanes of a row take a line each; never past the end of the half row)
+                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * rsA * sizeof(T) + row8_touch_offset(ln, h));
                 }
             }
         }

@@ -22,6 +22,7 @@
 #include <stddef.h>
 #include "../../include/mlstm_hip.h"
 #include "mlstm_device.h"
+#include "mlstm_kernels.h"
 
 namespace slstm {
 
@@ -432,21 +433,32 @@ int slices_for(int B, int NH, int S) {
     return (int)(n < 1 ? 1 : n);
 }
 
+// (the step kernels count their waits for the input ring by hand: see no_scratch_once)
+template <int DH, bool SAVE, bool FS>
+int forward_launch(const float* wx, const float* r, const float* b, float* h, float* saved, int B, int NH, int S, hipStream_t st) {
+    if (int rc = mlstm::no_scratch_once<slstm_forward_kernel<DH, SAVE, FS>>()) return rc;
+    hipLaunchKernelGGL((slstm_forward_kernel<DH, SAVE, FS>), dim3(B * NH), dim3(4 * DH), 0, st, wx, r, b, h, saved, NH, S);
+    return (int)hipGetLastError();
+}
+
 template <int DH>
 int forward_t(const float* wx, const float* r, const float* b, float* h, float* saved, int B, int NH, int S, int fs, hipStream_t st) {
-    const dim3 grid(B * NH), block(4 * DH);
-    if (saved && fs) hipLaunchKernelGGL((slstm_forward_kernel<DH, true, true>), grid, block, 0, st, wx, r, b, h, saved, NH, S);
-    else if (saved) hipLaunchKernelGGL((slstm_forward_kernel<DH, true, false>), grid, block, 0, st, wx, r, b, h, saved, NH, S);
-    else if (fs) hipLaunchKernelGGL((slstm_forward_kernel<DH, false, true>), grid, block, 0, st, wx, r, b, h, saved, NH, S);
-    else hipLaunchKernelGGL((slstm_forward_kernel<DH, false, false>), grid, block, 0, st, wx, r, b, h, saved, NH, S);
-    return (int)hipGetLastError();
+    if (saved && fs) return forward_launch<DH, true, true>(wx, r, b, h, saved, B, NH, S, st);
+    if (saved) return forward_launch<DH, true, false>(wx, r, b, h, saved, B, NH, S, st);
+    if (fs) return forward_launch<DH, false, true>(wx, r, b, h, saved, B, NH, S, st);
+    return forward_launch<DH, false, false>(wx, r, b, h, saved, B, NH, S, st);
 }
 
 template <int DH>
 int backward_t(const float* dh, const float* h, const float* r, const float* saved, float* dwx, float* dr, float* db, int B, int NH, int S,
                int fs, char* ws, hipStream_t st) {
-    if (fs) hipLaunchKernelGGL((slstm_backward_kernel<DH, true>), dim3(B * NH), dim3(4 * DH), 0, st, dh, r, saved, dwx, NH, S);
-    else hipLaunchKernelGGL((slstm_backward_kernel<DH, false>), dim3(B * NH), dim3(4 * DH), 0, st, dh, r, saved, dwx, NH, S);
+    if (fs) {
+        if (int rc = mlstm::no_scratch_once<slstm_backward_kernel<DH, true>>()) return rc;
+        hipLaunchKernelGGL((slstm_backward_kernel<DH, true>), dim3(B * NH), dim3(4 * DH), 0, st, dh, r, saved, dwx, NH, S);
+    } else {
+        if (int rc = mlstm::no_scratch_once<slstm_backward_kernel<DH, false>>()) return rc;
+        hipLaunchKernelGGL((slstm_backward_kernel<DH, false>), dim3(B * NH), dim3(4 * DH), 0, st, dh, r, saved, dwx, NH, S);
+    }
     const int ns = slices_for(B, NH, S);
     const size_t nr = (size_t)NH * 4 * DH * DH, nb = (size_t)NH * 4 * DH;
     float* part_r = reinterpret_cast<float*>(ws);
