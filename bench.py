@@ -379,6 +379,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-secondary", action="store_true", help="skip the secondary workloads (long context, scan, split mode)")
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
+    ap.add_argument("--chunk-length", type=int, default=0,
+                    help="measurement aid: chunk length of the 16-bit kernels (a multiple of 128; 0 = the library's choice, < 0 = no chunks)")
     ap.add_argument("--column-kernel", type=int, default=0, choices=[0, 1, 2, 3],
                     help="measurement aid: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -397,6 +399,7 @@ def main():
     global COLUMN_KERNEL
     COLUMN_KERNEL = args.column_kernel
     ffi.set_column_kernel(args.column_kernel)
+    ffi.set_chunk_length(args.chunk_length)
     if args.calibrate_copy:
         # 1 GiB, copied twice: four times the chip's 256 MB last-level cache, so the second copy's source comes from HBM
         # (a source that still sits in that cache reads as almost no FETCH_SIZE at all)

@@ -67,14 +67,9 @@ int chunk_len_for(int dtype, int D, size_t S) {
 // What mlstm_forward_save_* writes at the head of `saved` and mlstm_backward_saved_* checks on the device (no host
 // round trip): shape, types and the process-wide settings the two calls must agree on.
 constexpr size_t SAVED_HEADER_BYTES = 256;
-struct SavedHeader { int v[8]; };   // magic, BH, S, D, dtype argument, chunk length, kernel switch, states per head
+// The eight words: magic, BH, S, D, dtype argument, chunk length, kernel switch, states per head.  The forward's gate
+// pre-pass writes them and the backward's last kernel compares them (mlstm::SavedStamp): no launch of their own.
 constexpr int SAVED_MAGIC = 0x4d4c5356;   // "MLSV"
-__global__ void saved_header_write(int* dst, SavedHeader hd) {
-    if (threadIdx.x < 8) dst[threadIdx.x] = hd.v[threadIdx.x];
-}
-__global__ void saved_header_check(const int* src, SavedHeader hd, int* err) {
-    if (threadIdx.x < 8 && src[threadIdx.x] != hd.v[threadIdx.x]) atomicOr(err, 2);
-}
 
 struct Sizes {
     size_t BH, S, D, NG, el;
@@ -117,13 +112,14 @@ struct Sizes {
                up256(scan_segment_state_bytes((int)BH, (int)S, (int)D));
     }
     size_t fwd() const { return scan_engine() ? scan_fwd() : gates() + stats() + chunk_states(dtype_code); }
+    size_t anchor_parts() const { return D >= 64 ? (D / 64) * (D / 64) : 1; }   // workgroups per head of the value-major carry
     size_t fwd_fixed() const { return gates() + stats(); }   // offset of the chunk states inside fwd()
     size_t bwd() const {
         if (scan_engine()) return scan_backward_workspace_bytes((int)BH, (int)S, (int)D);
         return fwd() + up256(BH * S * D * el)                                      // recomputed h
                + 2 * up256(BH * NG * 64 * 4) + states_t()                          // inv_n, db; transposed chunk states
                + states_t() + saved_vec() + up256(BH * S * 4)                      // reverse states (value-major, vector); far row sums
-               + up256(BH * n_states(chunk_len()) * 4)                             // dF anchors
+               + up256(BH * n_states(chunk_len()) * anchor_parts() * 4)            // dF anchors (in parts)
                + up256(BH * S * 4) + up256(BH * row_slices() * S * 4)              // colsum, rowpart
                + h_lo();                                                           // split mode: low-order part of a recomputed h
     }
@@ -298,9 +294,12 @@ struct SavedView {
         if (z.precise) h_lo = p;
     }
 };
-SavedHeader saved_header_of(const Sizes& z) {
-    return SavedHeader{{SAVED_MAGIC, (int)z.BH, (int)z.S, (int)z.D, z.dtype_code | (z.precise ? MLSTM_PRECISE : 0), z.chunk_len(),
-                        mlstm::g_force_generic ? 1 : 0, (int)z.n_states(z.chunk_len())}};
+SavedStamp saved_stamp_of(const Sizes& z) {
+    SavedStamp s;
+    const int v[8] = {SAVED_MAGIC, (int)z.BH, (int)z.S, (int)z.D, z.dtype_code | (z.precise ? MLSTM_PRECISE : 0), z.chunk_len(),
+                      mlstm::g_force_generic ? 1 : 0, (int)z.n_states(z.chunk_len())};
+    for (int t = 0; t < 8; t++) s.v[t] = v[t];
+    return s;
 }
 
 // states at the chunk ends of a long sequence (both layouts when CstT is given; split mode: each as two terms, the
@@ -357,7 +356,8 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
                  const Sizes& z, int D, int dtype, int gate_dtype, char* ws, hipStream_t st, float** alpha_out = nullptr,
                  float** beta_out = nullptr, double** g_out = nullptr, float** m_out = nullptr, float** b_out = nullptr,
                  float** ek_out = nullptr, float** amax_out = nullptr, const void* o = nullptr, void* h_gated = nullptr,
-                 void* CstT = nullptr, float* Nst_ext = nullptr, char* gates_ext = nullptr, void* h_lo = nullptr) {
+                 void* CstT = nullptr, float* Nst_ext = nullptr, char* gates_ext = nullptr, void* h_lo = nullptr,
+                 const SavedStamp* stamp = nullptr) {
     if (z.scan_engine()) {
         // dense tensors only, no fused gate copy (mlstm_scan_forward_ex is the gated form of these kernels)
         if (o || h_gated || !is_dense(z.la, (long long)z.S, (long long)z.D) || !is_dense(z.lb, (long long)z.S, (long long)z.D)) return MLSTM_ESHAPE;
@@ -371,7 +371,7 @@ int forward_impl(const void* q, const void* k, const void* v, const void* f, con
     if (!b) b = w.bw;
     {
         Timed t(MLSTM_K_GATES, st);
-        hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st, z.lg, z.gate_form);
+        hipError_t e = launch_gates(gate_dtype, f, i, alpha2, beta2, G2, m, ek2, amax2, (int)z.BH, (int)z.S, st, z.lg, z.gate_form, stamp);
         if (e != hipSuccess) return (int)e;
     }
     RowArgs a{};
@@ -567,10 +567,10 @@ int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const voi
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     if (z.saved() == 0) return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st);
     SavedView sv((char*)saved, z);
-    hipLaunchKernelGGL(saved_header_write, dim3(1), dim3(64), 0, st, sv.header, saved_header_of(z));
-    if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+    SavedStamp stamp = saved_stamp_of(z);
+    stamp.dst = sv.header;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr,
-                        nullptr, nullptr, nullptr, sv.CstT, sv.Nst, sv.gates, sv.h_lo);
+                        nullptr, nullptr, nullptr, sv.CstT, sv.Nst, sv.gates, sv.h_lo, &stamp);
 }
 
 int mlstm_forward_gated_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
@@ -619,14 +619,14 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     const float* Nst = w.Nst;
     const bool reuse = saved && w.ncs > 0;
     const void* h_lo = nullptr;   // split mode: the low-order part of h, from the forward (saved) or from a recomputation
+    SavedStamp stamp;
     if (saved) {
         SavedView sv(const_cast<char*>(saved), z);
-        // the header is compared on the device: a buffer written for another shape, type or setting (chunk length, kernel
-        // switch) sets bit 1 of the error word, which mlstm_kernel_error reports
-        int* err = nullptr;
-        if (int rc = symbols_of_current_device(nullptr, &err)) return rc;
-        hipLaunchKernelGGL(saved_header_check, dim3(1), dim3(64), 0, st, sv.header, saved_header_of(z), err);
-        if (hipError_t e = hipGetLastError(); e != hipSuccess) return (int)e;
+        // the header is compared on the device (by the last kernel of this pass): a buffer written for another shape,
+        // type or setting (chunk length, kernel switch) sets bit 1 of the error word, which mlstm_kernel_error reports
+        stamp = saved_stamp_of(z);
+        stamp.src = sv.header;
+        if (int rc = symbols_of_current_device(nullptr, &stamp.err)) return rc;
         if (reuse) {   // the forward's states (value-major matrices, then the vectors) and its gate pre-pass
             CstT = sv.CstT;
             Nst = sv.Nst;
@@ -637,7 +637,8 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     char* Ev = c.take<char>(z.state_elems() * z.el * z.parts());    // reverse states, value-major
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
-    float* anchor = c.take<float>(z.BH * w.ncs);
+    float* anchor = c.take<float>(z.BH * w.ncs * z.anchor_parts());
+    const bool fused_anchor = w.L <= 1024;   // (the one-kernel dF pass adds the parts up; see DfArgs)
     char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
     const size_t lo_off = z.state_elems() * z.el;   // split mode: a set of states is [hi | lo]
     const bool col_chunks = z.col_chunks();
@@ -695,8 +696,10 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         ra2.lk = z.la; ra2.lv = z.lb;
         ra2.precise = z.precise ? 1 : 0;
         ra2.CstT_lo = z.precise ? Ev + lo_off : nullptr;
+        if (fused_anchor) { ra2.dot_with = CstT; ra2.dot_with_lo = z.precise ? CstT + lo_off : nullptr; ra2.dot_part = anchor; }
         if (int e = launch_chunk_states(dtype, D, ra2, st)) return e;
-        if (int e = launch_anchor(dtype, D, CstT, Ev, z.precise ? CstT + lo_off : nullptr, z.precise ? Ev + lo_off : nullptr, Nst, gvec, anchor,
+        if (fused_anchor) {
+        } else if (int e = launch_anchor(dtype, D, CstT, Ev, z.precise ? CstT + lo_off : nullptr, z.precise ? Ev + lo_off : nullptr, Nst, gvec, anchor,
                                   (int)z.BH, (int)w.ncs, st))
             return e;   // (both value-major)
     }
@@ -713,7 +716,10 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     }
 
     DfArgs da{f, colsum, rowpart, df, di, (int)z.BH, (int)z.S, (int)z.NG, (int)z.row_slices(), col_chunks ? w.L : 0, rowinter, anchor, (int)w.ncs};
-    da.lg = z.lg; da.gate_form = z.gate_form;
+    da.lg = z.lg; da.gate_form = z.gate_form; da.stamp = stamp;
+    if (col_chunks && fused_anchor) {
+        da.anchor = nullptr; da.anchor_part = anchor; da.anchor_parts = (int)z.anchor_parts(); da.anchor_va = Nst; da.anchor_vb = gvec; da.D = D;
+    }
     Timed t(MLSTM_K_DF, st);
     return launch_df(gate_dtype, da, st);
 }

@@ -12,7 +12,9 @@ namespace mlstm {
 // slices at or below the position's own tile), the four partial sums meet in LDS.
 template <typename TG>
 __global__ __launch_bounds__(256) void rowreduce_kernel(const float* __restrict__ colsum, float* rowpart, TG* __restrict__ dI,
-                                                        int S, int NG, int RS, int chunk_tiles, const float* __restrict__ rowinter, Lay lg) {
+                                                        int S, int NG, int RS, int chunk_tiles, const float* __restrict__ rowinter, Lay lg,
+                                                        SavedStamp stamp) {
+    stamp_apply(stamp, blockIdx.x == 0 && blockIdx.y == 0, threadIdx.x);
     __shared__ float part[4][GRAN];
     const int bh = blockIdx.y, g = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int t = GRAN * g + lane, tc = t < S ? t : S - 1;
@@ -97,9 +99,30 @@ template <typename TG>
 __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F, const float* __restrict__ colsum, const float* __restrict__ rowpart,
                                                        const float* __restrict__ rowinter, const float* __restrict__ anchor,
                                                        TG* __restrict__ dF, TG* __restrict__ dI, int S, int RS, int chunk_len, int n_states,
-                                                       Lay lg, int form) {
+                                                       Lay lg, int form, const float* __restrict__ anchor_part, int anchor_parts,
+                                                       const float* __restrict__ va, const float* __restrict__ vb, int D, SavedStamp stamp) {
     __shared__ float wt[16];
+    __shared__ float at[2][16];
     const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    stamp_apply(stamp, c == 0 && bh == 0, tid);
+    // the two anchors of this chunk (its first position, and the next chunk's) from their parts: the partial sums of the
+    // matrix states' contraction and the product of the vector states; both states carry the factor 1 / sqrt(D) of the
+    // scores, dD has it once
+    float a_start = 0.f, a_next = 0.f;
+    if (anchor_part) {
+#pragma unroll
+        for (int w = 0; w < 2; w++) {
+            const int cs = c - 1 + w;
+            float x = 0.f;
+            if (cs >= 0 && cs < n_states) {
+                const size_t o = (size_t)bh * n_states + cs;
+                if (tid < D) x = va[o * D + tid] * vb[o * D + tid];
+                if (tid < anchor_parts) x += anchor_part[o * anchor_parts + tid];
+            }
+            x = wave_scan_inclusive<OpAdd>(x);
+            if (lane == 63) at[w][wave] = x;
+        }
+    }
     const int t = c * chunk_len + tid;
     const bool live = tid < chunk_len && t < S;
     float v = 0.f, col = 0.f, f = 0.f;
@@ -122,9 +145,18 @@ __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F,
         if (w < wave) pre += s;
         tot += s;
     }
-    const float start = c > 0 ? anchor[(size_t)bh * n_states + c - 1] : 0.f;
+    if (anchor_part) {
+        const float rs = sqrtf((float)D);
+#pragma unroll
+        for (int w = 0; w < 16; w++) { a_start += at[0][w]; a_next += at[1][w]; }
+        a_start *= rs; a_next *= rs;
+    } else {
+        a_start = c > 0 ? anchor[(size_t)bh * n_states + c - 1] : 0.f;
+        a_next = c < n_states ? anchor[(size_t)bh * n_states + c] : 0.f;
+    }
+    const float start = c > 0 ? a_start : 0.f;
     // what the chunk's own (rounded) sums miss of the next anchor is spread evenly over its positions
-    const float bridge = c < n_states ? (anchor[(size_t)bh * n_states + c] - (start + tot)) / (float)chunk_len : 0.f;
+    const float bridge = c < n_states ? (a_next - (start + tot)) / (float)chunk_len : 0.f;
     if (live) {
         const float excl = start + (pre + (incl - v)) + bridge * (float)tid;
         dF[lg.head(bh) + (size_t)t * lg.ss] = (TG)forget_grad(form, f, excl, v, t);
@@ -137,11 +169,12 @@ static int launch_df_t(const DfArgs& a, hipStream_t st) {
     if (a.chunk_len > 0 && a.chunk_len <= 1024) {
         hipLaunchKernelGGL(dfchunk_kernel<TG>, dim3((a.S + a.chunk_len - 1) / a.chunk_len, a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F),
                            a.colsum, a.rowpart, a.rowinter, a.anchor, reinterpret_cast<TG*>(a.dF), reinterpret_cast<TG*>(a.dI), a.S, a.RS,
-                           a.chunk_len, a.n_states, a.lg, a.gate_form);
+                           a.chunk_len, a.n_states, a.lg, a.gate_form, a.anchor_part, a.anchor_parts, a.anchor_va, a.anchor_vb, a.D, a.stamp);
         return (int)hipGetLastError();
     }
+    if (a.anchor_part) return MLSTM_EINVAL;   // (only the one-kernel form adds the parts up)
     hipLaunchKernelGGL(rowreduce_kernel<TG>, dim3((a.S + GRAN - 1) / GRAN, a.BH), dim3(256), 0, st, a.colsum, const_cast<float*>(a.rowpart),
-                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.RS, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr, a.lg);
+                       reinterpret_cast<TG*>(a.dI), a.S, a.NG, a.RS, a.chunk_len / GRAN, a.chunk_len > 0 ? a.rowinter : nullptr, a.lg, a.stamp);
     hipLaunchKernelGGL(dfscan_kernel<TG>, dim3(a.BH), dim3(1024), 0, st, reinterpret_cast<const TG*>(a.F), a.rowpart,
                        reinterpret_cast<TG*>(a.dF), a.S, a.RS, a.chunk_len, a.anchor, a.n_states, a.lg, a.gate_form);
     return (int)hipGetLastError();

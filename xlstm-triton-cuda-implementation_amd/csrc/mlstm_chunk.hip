@@ -400,6 +400,11 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
         const f32x4 d1 = *reinterpret_cast<const f32x4*>(src + (size_t)c * D * D + 4);
         run0 = run0 * gam + d0;
         run1 = run1 * gam + d1;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {   // (see chunk_carry_t_kernel: the fp32 value is fixed before any conversion)
+            asm volatile("" : "+v"(run0[e]));
+            asm volatile("" : "+v"(run1[e]));
+        }
         if (a.Cst && !a.CstT) {   // (with a value-major copy wanted, chunk_carry_t_kernel writes both layouts)
             typedef typename Tr<T>::vec4 V4;
             struct Pair { V4 lo, hi; };
@@ -426,8 +431,8 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
 // value index): a workgroup takes 64 values x 64 keys, reads the chunk sums along the value index (coalesced), and
 // turns the block round in LDS so that the rows leave 128 bytes at a time.  Rows in the contraction order of the row
 // kernel, like the untransposed states.
-template <typename T, int D>
-__global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
+template <typename T, int D, bool DOT, bool KM>
+__global__ __launch_bounds__(256, 4) void chunk_carry_t_kernel(ChunkArgs a) {
     __shared__ __attribute__((aligned(16))) T tile[2][64][64 + 8];   // [hi | lo (split mode)]
     const int bh = blockIdx.y, tid = threadIdx.x;
     const bool split = a.CstT_lo != nullptr;
@@ -446,6 +451,10 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
     float* nst = a.Nst + (size_t)bh * a.NCS * D + tid;   // the vector states, in place, by the first workgroup of a head
     const bool vec = blockIdx.x == 0 && tid < D;
     float nrun = 0.f;
+    __shared__ float red[4];
+    const int lane = tid & 63, wave = tid >> 6;
+    // (the kernel moves 4 bytes in and 2 to 4 out per element and runs at memory speed: nothing to gain from requesting a
+    // step's chunk sums ahead of time)
     for (int step = 0; step < a.NCS; step++) {
         const int c = a.reverse ? a.NCS - 1 - step : step;
         const float gam = step > 0 ? carry_gamma(a, poff, goff, a.reverse ? c + 1 : c) : 0.f;
@@ -454,13 +463,19 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
             nst[(size_t)c * D] = nrun;
         }
         const float* src = a.dC + ((size_t)bh * a.NCS + c) * D * D + 64 * vb + vl;
+        typedef typename Tr<T>::frag V8;
 #pragma unroll
         for (int g = 0; g < 2; g++) {
             f32x8 d;
 #pragma unroll
             for (int e = 0; e < 8; e++) d[e] = src[(size_t)(64 * kb + 8 * (kq + 4 * g) + e) * D];
             run[g] = run[g] * gam + d;
-            if (a.Cst) {   // key-major copy: lanes of a wave hold consecutive values of one key, 128 bytes per store
+            // (the fp32 value is fixed here: left to itself the compiler may fold this multiply-add into a conversion to
+            // fp16 further down -- one rounding instead of two -- in one kernel and not in its twin, and the two carries
+            // must give the same bits)
+#pragma unroll
+            for (int e = 0; e < 8; e++) asm volatile("" : "+v"(run[g][e]));
+            if constexpr (KM) {   // key-major copy: lanes of a wave hold consecutive values of one key, 128 bytes per store
                 const size_t koff = ((size_t)bh * a.NCS + c) * D * D + 64 * vb + vl;
                 T* kd = reinterpret_cast<T*>(a.Cst) + koff;
 #pragma unroll
@@ -489,12 +504,36 @@ __global__ __launch_bounds__(256) void chunk_carry_t_kernel(ChunkArgs a) {
         const uint4 p0 = *reinterpret_cast<const uint4*>(&tile[0][orow][16 * opiece]), p1 = *reinterpret_cast<const uint4*>(&tile[0][orow][16 * opiece + 8]);
         *reinterpret_cast<uint4*>(dst + (size_t)c * D * D) = p0;
         *reinterpret_cast<uint4*>(dst + (size_t)c * D * D + 8) = p1;
+        if constexpr (DOT) {   // <state c as it is written (the sum of its terms in split mode), the other set's state c>
+            f32x8 x0 = __builtin_convertvector(__builtin_bit_cast(V8, p0), f32x8), x1 = __builtin_convertvector(__builtin_bit_cast(V8, p1), f32x8);
+            // the other set's state c at the places this thread has just written (four workgroups share a CU: their
+            // steps hide this round trip)
+            const size_t doff = (size_t)(dst - reinterpret_cast<T*>(a.CstT)) + (size_t)c * D * D;
+            const T* other = reinterpret_cast<const T*>(a.dot_with) + doff;
+            f32x8 y0 = __builtin_convertvector(*reinterpret_cast<const V8*>(other), f32x8);
+            f32x8 y1 = __builtin_convertvector(*reinterpret_cast<const V8*>(other + 8), f32x8);
+            if (split) {
+                x0 += __builtin_convertvector(*reinterpret_cast<const V8*>(&tile[1][orow][16 * opiece]), f32x8);
+                x1 += __builtin_convertvector(*reinterpret_cast<const V8*>(&tile[1][orow][16 * opiece + 8]), f32x8);
+            }
+            if (a.dot_with_lo) {
+                const T* other_lo = reinterpret_cast<const T*>(a.dot_with_lo) + doff;
+                y0 += __builtin_convertvector(*reinterpret_cast<const V8*>(other_lo), f32x8);
+                y1 += __builtin_convertvector(*reinterpret_cast<const V8*>(other_lo + 8), f32x8);
+            }
+            const f32x8 pr = x0 * y0 + x1 * y1;
+            float dot = ((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7]));
+            dot = wave_scan_inclusive<OpAdd>(dot);
+            if (lane == 63) red[wave] = dot;
+        }
         if (split) {
             T* dlo = reinterpret_cast<T*>(a.CstT_lo) + (dst - reinterpret_cast<T*>(a.CstT));
             *reinterpret_cast<uint4*>(dlo + (size_t)c * D * D) = *reinterpret_cast<const uint4*>(&tile[1][orow][16 * opiece]);
             *reinterpret_cast<uint4*>(dlo + (size_t)c * D * D + 8) = *reinterpret_cast<const uint4*>(&tile[1][orow][16 * opiece + 8]);
         }
         __syncthreads();
+        if (DOT && tid == 0)   // (the waves' sums were written between the two barriers; the next ones follow the next barrier)
+            a.dot_part[((size_t)bh * a.NCS + c) * gridDim.x + blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
     }
 }
 
@@ -522,7 +561,14 @@ static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     if (a.precise && ((a.Cst && !a.Cst_lo) || (a.CstT && !a.CstT_lo))) return MLSTM_EINVAL;
     if (int rc = a.precise ? launch_chunk_sum<T, D, true>(a, st) : launch_chunk_sum<T, D, false>(a, st)) return rc;
     // one carry kernel: the value-major one writes both layouts and the vector states
-    if (a.CstT) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D>), dim3((D / 64) * (D / 64), a.BH), dim3(256), 0, st, a);
+    if (a.dot_part && !(a.CstT && a.dot_with)) return MLSTM_EINVAL;
+    // (the variants of the value-major carry: with the contraction, with the key-major copy, with neither; both at once do
+    // not fit the registers of four workgroups per CU, and nothing asks for both)
+    const dim3 cgrid((D / 64) * (D / 64), a.BH);
+    if (a.CstT && a.dot_part && a.Cst) return MLSTM_EINVAL;
+    else if (a.CstT && a.dot_part) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D, true, false>), cgrid, dim3(256), 0, st, a);
+    else if (a.CstT && a.Cst) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D, false, true>), cgrid, dim3(256), 0, st, a);
+    else if (a.CstT) hipLaunchKernelGGL((chunk_carry_t_kernel<T, D, false, false>), cgrid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((chunk_carry_kernel<T, D>), dim3(D * D / 8 / 256, a.BH), dim3(256), 0, st, a);
     return (int)hipGetLastError();
 }

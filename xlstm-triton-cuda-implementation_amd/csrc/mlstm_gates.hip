@@ -87,7 +87,9 @@ __device__ __forceinline__ float forget_log(const TG* f, size_t ss, int t, int f
 template <typename TG, int GPW>
 __global__ __launch_bounds__(1024) void gates_kernel_reg(const TG* __restrict__ F, const TG* __restrict__ I, float* __restrict__ alpha2,
                                                         float* __restrict__ beta2, double* __restrict__ G2, float* __restrict__ M,
-                                                        float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form) {
+                                                        float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form,
+                                                        SavedStamp stamp) {
+    stamp_apply(stamp, blockIdx.x == 0, threadIdx.x);
     __shared__ double sT[16 * GPW];
     __shared__ double sP[16 * GPW];
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -128,7 +130,9 @@ __global__ __launch_bounds__(1024) void gates_kernel_reg(const TG* __restrict__ 
 template <typename TG>
 __global__ __launch_bounds__(1024) void gates_kernel(const TG* __restrict__ F, const TG* __restrict__ I, float* __restrict__ alpha2,
                                                     float* __restrict__ beta2, double* __restrict__ G2, float* __restrict__ M,
-                                                    float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form) {
+                                                    float* __restrict__ ek2, float* __restrict__ amax2, int S, int NG, Lay lg, int form,
+                                                    SavedStamp stamp) {
+    stamp_apply(stamp, blockIdx.x == 0, threadIdx.x);
     __shared__ double sT[GATES_MAX_GRANULES];  // granule totals of lf, then exclusive prefix G
     __shared__ double sP[GATES_MAX_GRANULES];  // granule maxima of alpha, then running max R of (P - G) over earlier granules
     const int bh = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -164,25 +168,26 @@ __global__ __launch_bounds__(1024) void gates_kernel(const TG* __restrict__ F, c
 
 template <typename TG>
 static hipError_t launch_gates_t(const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                                 float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form) {
+                                 float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form, const SavedStamp& stamp) {
     int NG = (S + GRAN - 1) / GRAN;
     if (NG <= 16 * 4)
-        hipLaunchKernelGGL((gates_kernel_reg<TG, 4>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
+        hipLaunchKernelGGL((gates_kernel_reg<TG, 4>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     else if (NG <= 16 * 8)
-        hipLaunchKernelGGL((gates_kernel_reg<TG, 8>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
+        hipLaunchKernelGGL((gates_kernel_reg<TG, 8>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     else
-        hipLaunchKernelGGL(gates_kernel<TG>, dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form);
+        hipLaunchKernelGGL(gates_kernel<TG>, dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     return hipGetLastError();
 }
 
 hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form) {
+                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int form, const SavedStamp* stamp_in) {
+    const SavedStamp stamp = stamp_in ? *stamp_in : SavedStamp{};
     if ((S + GRAN - 1) / GRAN > GATES_MAX_GRANULES) return hipErrorInvalidValue;
     if (form == MLSTM_GATE_CUMSUM && gate_dtype != MLSTM_F32) return hipErrorInvalidValue;   // (16-bit types cannot hold the sum)
     switch (gate_dtype) {
-        case MLSTM_F32: return launch_gates_t<float>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
-        case MLSTM_F16: return launch_gates_t<_Float16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
-        case MLSTM_BF16: return launch_gates_t<__bf16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form);
+        case MLSTM_F32: return launch_gates_t<float>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form, stamp);
+        case MLSTM_F16: return launch_gates_t<_Float16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form, stamp);
+        case MLSTM_BF16: return launch_gates_t<__bf16>(F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, lg, form, stamp);
     }
     return hipErrorInvalidValue;
 }

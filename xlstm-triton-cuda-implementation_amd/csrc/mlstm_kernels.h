@@ -44,12 +44,28 @@ inline Lay dense_layout(int NH, long long S, long long D) { return Lay{(long lon
 // strides cost them address arithmetic in loops that are bound by instruction issue.)
 inline bool is_dense(const Lay& l, long long S, long long D) { return l.ss == D && l.sh == S * D && l.sb == (long long)l.NH * S * D; }
 
+// Eight words that one kernel of the forward leaves at the head of a caller-kept buffer (dst) and one kernel of the backward
+// compares with what it finds there (src; a difference sets bit 1 of *err): rides along in kernels that run anyway.
+struct SavedStamp {
+    int* dst = nullptr;
+    const int* src = nullptr;
+    int* err = nullptr;
+    int v[8] = {};
+};
+#if defined(__HIPCC__)
+__device__ __forceinline__ void stamp_apply(const SavedStamp& s, bool first_block, int tid) {
+    if (!first_block || tid >= 8) return;
+    if (s.dst) s.dst[tid] = s.v[tid];
+    if (s.src && s.src[tid] != s.v[tid]) atomicOr(s.err, 2);
+}
+#endif
+
 // Gate pre-pass: alpha2, beta2 [BH, NG*64] fp32 (NG = ceil(S/64), rows padded), G2 [BH, NG] fp64, M [BH,S] fp32.
 // ek2 [BH, NG*64] = exp2(alpha2 - block max), amax2 [BH, NG*2] = the maxima of alpha2 over blocks of 32 positions.
 // lg: layout of F and I.  gate_form: what F holds (MLSTM_GATE_RAW: the forget gate's pre-activation, _LOGSIGMOID: its
 // log-sigmoid, _CUMSUM: the cumulative sum of that over the positions of a head).
 hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
-                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int gate_form);
+                        float* amax2, int BH, int S, hipStream_t st, const Lay& lg, int gate_form, const SavedStamp* stamp = nullptr);
 inline hipError_t launch_gates(int gate_dtype, const void* F, const void* I, float* alpha2, float* beta2, double* G2, float* M, float* ek2,
                                float* amax2, int BH, int S, hipStream_t st) {
     return launch_gates(gate_dtype, F, I, alpha2, beta2, G2, M, ek2, amax2, BH, S, st, dense_layout(BH, S, 1), MLSTM_GATE_RAW);
@@ -171,6 +187,14 @@ struct DfArgs {
     int n_states;
     Lay lg;                  // layout of F, dF and dI
     int gate_form;           // what F holds (see launch_gates); dF is the gradient of that same quantity
+    // chunk_len <= 1024: the anchors come as partial sums instead (ChunkArgs::dot_part of the reverse states) and the
+    // vector states of both directions, and the kernel adds them up itself
+    const float* anchor_part = nullptr;   // [BH][n_states][anchor_parts]
+    int anchor_parts = 0;
+    const float* anchor_va = nullptr;     // [BH][n_states][D] each
+    const float* anchor_vb = nullptr;
+    int D = 0;
+    SavedStamp stamp;        // compared by the first workgroup (src), if set
 };
 int launch_df(int gate_dtype, const DfArgs& a, hipStream_t st);
 
@@ -199,6 +223,12 @@ struct ChunkArgs {
     int precise;
     void* Cst_lo;
     void* CstT_lo;
+    // The value-major carry can contract the states it forms (before rounding) with another set in the same layout
+    // (dot_with, dot_with_lo: its low-order terms or null): dot_part[bh][c][workgroup of the head] receives the partial
+    // sums of <state_c, dot_with_c>, (D / 64)^2 per state.
+    const void* dot_with = nullptr;
+    const void* dot_with_lo = nullptr;
+    float* dot_part = nullptr;
 };
 int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st);
 
