@@ -31,6 +31,9 @@ WORKLOADS = {
     "cfg2_B1_H4_S2048_D64_f32": (1, 4, 2048, 64, torch.float32, 0.0, 0.0, 1.0),
     "aux_B4_H16_S4096_D128_bf16": (4, 16, 4096, 128, torch.bfloat16, 3.0, 0.0, 1.0),
     "aux_B4_H8_S4096_D256_f16": (4, 8, 4096, 256, torch.float16, 3.0, 0.0, 1.0),
+    "aux_B4_H8_S4096_D64_bf16": (4, 8, 4096, 64, torch.bfloat16, 3.0, 0.0, 1.0),
+    "aux_B2_H8_S4096_D128_f32": (2, 8, 4096, 128, torch.float32, 3.0, 0.0, 1.0),
+    "aux_B4_H8_S4096_D64_f32": (4, 8, 4096, 64, torch.float32, 3.0, 0.0, 1.0),
 }
 COLUMN_KERNEL = 0   # --column-kernel
 PEAK_TFLOPS = {torch.bfloat16: 2500.0, torch.float16: 2500.0, torch.float32: 157.3}

@@ -190,3 +190,66 @@ def test_chunked_forward_at_the_headline_shape():
         d = h.float() - h0.float()
         assert float(d.pow(2).mean().sqrt() / h0.float().pow(2).mean().sqrt()) < 2e-3, L
         assert float((b - b0).pow(2).mean().sqrt() / b0.pow(2).mean().sqrt()) < 1e-5, L
+
+
+SMALL = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.mark.parametrize("dt,S,D,L", [("f32", 1100, 64, 128), ("f32", 2048, 64, 0), ("f32", 900, 128, 256), ("f32", 1300, 128, 0),
+                                      ("bf16", 1100, 64, 128), ("f16", 2048, 64, 0), ("bf16", 1500, 64, 0), ("f16", 700, 64, 256)])
+def test_small_shapes_in_chunks(dt, S, D, L):
+    # fp32 (D = 64, 128) and the 16-bit types at D = 64: chunk sums by plain multiply-adds, one carry for both state
+    # layouts, the four-wave tile kernels in chunk mode.  fp32 is held to its own bound (every element, rtol 1e-4).
+    dtype = SMALL[dt]
+    q, k, v, f, i, dh = O.make_inputs(1, 2, S, D, dtype, seed=S + D + L + 5, f_mean=2.0)
+    args = dev(dh, q, k, v, f, i)
+    Lc = length_in_use(L, S, D, dtype)
+    assert Lc > 0 and (L == 0 or Lc == L)
+    with chunk_length(L):
+        h, m, b, saved = mm.mlstm_forward_save_hip(*args[1:])
+        assert saved is not None
+        got = mm.mlstm_backward_saved_hip(*args, h, m, b, saved)
+        again = mm.mlstm_backward_hip(*args, h, m, b)            # forms the states again
+        h2, m2, b2 = mm.mlstm_forward_hip(*args[1:])
+    assert torch.equal(h, h2) and torch.equal(m, m2) and torch.equal(b, b2)
+    for name, a, w in zip(["dq", "dk", "dv", "df", "di"], got, again):
+        assert torch.equal(a, w), name
+    assert_matches_oracle(dtype, q, k, v, f, i, dh, h=h, m=m, b=b, grads=got, chunk_len=Lc)
+    with chunk_length(-1):
+        h0, m0, b0 = mm.mlstm_forward_hip(*args[1:])
+        plain = mm.mlstm_backward_hip(*args, h0, m0, b0)
+    assert torch.equal(m, m0)
+    sig = combined(rounding_noise(dh, q, k, v, f, i, dtype), rounding_noise(dh, q, k, v, f, i, dtype, chunk_len=Lc)) if dtype != torch.float32 else None
+    for name, g, p in zip(["h", "dq", "dk", "dv", "df", "di"], [h, *got], [h0, *plain]):
+        assert_close(g, p.float(), dtype, name + " chunked vs unchunked", sig[name] if sig else None)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+def test_split_mode_in_chunks_at_head_dimension_64(dt):
+    # split mode at D = 64: two-term states from the element-wise carry, the literal bound
+    dtype = SMALL[dt]
+    S, D = 1100, 64
+    q, k, v, f, i, dh = O.make_inputs(1, 2, S, D, dtype, seed=411, f_mean=2.0)
+    args = dev(dh, q, k, v, f, i)
+    with chunk_length(256):
+        h, m, b, saved = mm.mlstm_forward_save_hip(*args[1:], precise=True)
+        got = mm.mlstm_backward_saved_hip(*args, h, m, b, saved, precise=True)
+    assert_matches_oracle(dtype, q, k, v, f, i, dh, h=h, m=m, b=b, grads=got, chunk_len=256, precise=True)
+
+
+def test_fp32_default_chunk_length_and_many_heads():
+    # the default for fp32 is the shortest chunk; a batch of heads gives the bits of its heads run alone
+    assert length_in_use(0, 2048, 64, torch.float32) == 128 and length_in_use(0, 1023, 64, torch.float32) == 0
+    assert length_in_use(0, 4096, 64, torch.bfloat16) == 256 and length_in_use(0, 4096, 128, torch.bfloat16) == 512
+    g = torch.Generator(device="cuda").manual_seed(5)
+    B, NH, S, D = 2, 3, 1536, 64
+    q, k, v, dh = (torch.randn(B, NH, S, D, generator=g, device="cuda") for _ in range(4))
+    f, i = torch.randn(B, NH, S, generator=g, device="cuda") + 3.0, torch.randn(B, NH, S, generator=g, device="cuda")
+    h, m, b, saved = mm.mlstm_forward_save_hip(q, k, v, f, i)
+    grads = mm.mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved)
+    one = [x[1:2, 2:3].contiguous() for x in (dh, q, k, v, f, i)]
+    h1, m1, b1, s1 = mm.mlstm_forward_save_hip(*one[1:])
+    g1 = mm.mlstm_backward_saved_hip(*one, h1, m1, b1, s1)
+    assert torch.equal(h1[0, 0], h[1, 2]) and torch.equal(b1[0, 0], b[1, 2])
+    for name, a, w in zip(["dq", "dk", "dv", "df", "di"], g1, grads):
+        assert torch.equal(a[0, 0], w[1, 2]), name

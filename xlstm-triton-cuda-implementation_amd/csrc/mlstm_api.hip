@@ -57,11 +57,17 @@ struct Carver {
 // states cost 2 S D^2 flops per head whatever the length.
 int g_chunk_override = 0;   // test aid: > 0 forces this length, < 0 switches chunking off
 int chunk_len_for(int dtype, int D, size_t S) {
-    // (the chunk states are formed by 16-bit MFMA products at D = 128 and 256; every tile kernel of those types knows
-    // chunks, the four-wave ones of split mode and of the test switch included)
-    if (dtype == MLSTM_F32 || !(D == 128 || D == 256) || g_chunk_override < 0) return 0;
+    // (the chunk states are formed by 16-bit MFMA products at D = 128 and 256 and by plain multiply-adds at the smaller
+    // shapes; every tile kernel knows chunks, the four-wave ones of fp32, of split mode and of the test switch included)
+    const bool shape_ok = dtype == MLSTM_F32 ? (D == 64 || D == 128) : (D == 64 || D == 128 || D == 256);
+    if (!shape_ok || g_chunk_override < 0) return 0;
     if (g_chunk_override > 0) return S > (size_t)g_chunk_override ? g_chunk_override : 0;
-    return S >= 1024 ? 512 : 0;   // (below two full chunks the state pass costs more than the skipped key tiles)
+    if (S < 1024) return 0;   // (below two full chunks of 512 the state pass costs more than the skipped key tiles)
+    // fp32 products run at a sixteenth of the 16-bit rate, so the key tiles a chunk saves weigh more against the states: the
+    // shortest chunk wins there (B1 H4 S2048 D64: 0.47 ms unchunked, 0.24 / 0.16 / 0.13 ms at 512 / 256 / 128; D = 128
+    // likewise); at D = 64 in 16 bits 256 is the measured best (B4 H8 S4096: 0.48 unchunked, 0.24 / 0.22 / 0.25 ms)
+    if (dtype == MLSTM_F32) return 128;
+    return D == 64 ? 256 : 512;
 }
 
 // What mlstm_forward_save_* writes at the head of `saved` and mlstm_backward_saved_* checks on the device (no host
@@ -638,7 +644,8 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs * z.anchor_parts());
-    const bool fused_anchor = w.L <= 1024;   // (the one-kernel dF pass adds the parts up; see DfArgs)
+    // (the one-kernel dF pass adds the parts up; see DfArgs)
+    const bool fused_anchor = w.L <= 1024 && mlstm::chunk_states_fused_dot(dtype, D);
     char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
     const size_t lo_off = z.state_elems() * z.el;   // split mode: a set of states is [hi | lo]
     const bool col_chunks = z.col_chunks();

@@ -27,6 +27,9 @@ namespace mlstm {
 // tile hands it rows 16 s + 4 h + e (e < 4) and 16 s + 8 + 4 h + e - 4 (e >= 4).  Tile row u (mod 16) therefore holds
 // state row PERM16(u): the two middle groups of four swap places.
 __device__ __forceinline__ int perm16(int u) { return (u & ~12) | ((u & 4) << 1) | ((u & 8) >> 1); }
+// (fp32 tiles are read one element per lane, in the natural order)
+template <typename T>
+__device__ __forceinline__ int state_row(int u) { return sizeof(T) == 2 ? ((u & ~15) | perm16(u & 15)) : u; }
 
 // STRICT: split mode, the weighted V rows go to LDS as two tiles, hi and lo (ChunkArgs::precise)
 template <typename T, int D, bool STRICT = false>
@@ -372,6 +375,87 @@ __global__ __launch_bounds__(512) void chunk_sum_kernel(ChunkArgs a) {
 #endif
 }
 
+// The chunk sums for the shapes the MFMA kernel above does not serve (fp32 at D = 64 and 128, 16-bit types at D = 64): the
+// same sums as plain fp32 multiply-adds out of LDS tiles of 64 positions.  One workgroup per (head, chunk, 64 value
+// columns); a thread holds D/16 keys x 4 values.  These shapes are small (the sums are 2 S D^2 flops per head).
+template <typename T, int D>
+__global__ __launch_bounds__(256) void chunk_sum_small_kernel(ChunkArgs a) {
+    constexpr int VW = 64, VH = D / VW, KPT = D / 16;
+    __shared__ __attribute__((aligned(16))) float ks[GRAN][D + 4];
+    __shared__ __attribute__((aligned(16))) float vs[GRAN][VW + 4];
+    __shared__ float sw2[GRAN];
+    const int tid = threadIdx.x;
+    const int vh = blockIdx.x % VH, pair = blockIdx.x / VH;
+    const int cc = pair % a.NCS, bh = pair / a.NCS;
+    const int S = a.S, L = a.L;
+    const size_t poff = (size_t)bh * a.NG * GRAN, goff = (size_t)bh * a.NG;
+    // (the positions and the reference point of a sum: see chunk_sum_kernel)
+    const int p0 = (a.reverse ? cc + 1 : cc) * L, pe = a.reverse ? p0 - 1 : p0 + L - 1;
+    const size_t rsK = (size_t)a.lk.ss, rsV = (size_t)a.lv.ss;
+    const T* Kh = reinterpret_cast<const T*>(a.K) + a.lk.head(bh);
+    const T* Vh = reinterpret_cast<const T*>(a.V) + a.lv.head(bh) + VW * vh;
+    const float log2scale = -0.5f * __log2f((float)D);
+    const float bend = a.beta2[poff + pe];
+    const double Gend = a.G2[goff + pe / GRAN];
+    const int k0 = KPT * (tid >> 4), v0 = 4 * (tid & 15);
+    float acc[KPT][4];
+#pragma unroll
+    for (int x = 0; x < KPT; x++)
+#pragma unroll
+        for (int y = 0; y < 4; y++) acc[x][y] = 0.f;
+    float nacc = 0.f;
+    const int n_pos = (p0 + L <= S ? L : S - p0);
+    for (int t0 = 0; t0 < n_pos; t0 += GRAN) {
+        __syncthreads();   // (the previous tile has been used)
+        // position tid / 4 of the tile, a quarter of its row each: K as it is, V times the position's weight
+        {
+            const int j = tid >> 2, part = tid & 3;
+            const int pos = p0 + t0 + j, pc = pos < S ? pos : S - 1;
+            float w = 0.f, w2 = 0.f;
+            if (pos < S) {
+                if (a.reverse) {
+                    const float rho = fast_exp2(bend - a.beta2[poff + pos] + (float)(a.G2[goff + pos / GRAN] - Gend) + log2scale);
+                    w = rho * a.inv_n[poff + pos];
+                    w2 = rho * a.db[poff + pos];
+                } else {
+                    w = w2 = fast_exp2(a.alpha2[poff + pos] - bend + (float)(Gend - a.G2[goff + pos / GRAN]) + log2scale);
+                }
+            }
+            if (part == 0) sw2[j] = w2;
+            const T* kr = Kh + (size_t)pc * rsK + (D / 4) * part;
+            const T* vr = Vh + (size_t)pc * rsV + (VW / 4) * part;
+#pragma unroll
+            for (int e = 0; e < D / 4; e++) ks[j][(D / 4) * part + e] = (float)kr[e];
+#pragma unroll
+            for (int e = 0; e < VW / 4; e++) vs[j][(VW / 4) * part + e] = (float)vr[e] * w;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int j = 0; j < GRAN; j++) {
+            const f32x4 vv = *reinterpret_cast<const f32x4*>(&vs[j][v0]);
+            float kk[KPT];
+#pragma unroll
+            for (int x = 0; x < KPT; x += 4) {
+                const f32x4 q4 = *reinterpret_cast<const f32x4*>(&ks[j][k0 + x]);
+                kk[x] = q4[0]; kk[x + 1] = q4[1]; kk[x + 2] = q4[2]; kk[x + 3] = q4[3];
+            }
+#pragma unroll
+            for (int x = 0; x < KPT; x++)
+#pragma unroll
+                for (int y = 0; y < 4; y++) acc[x][y] += kk[x] * vv[y];
+        }
+        if (vh == 0 && tid < D) {
+#pragma unroll 8
+            for (int j = 0; j < GRAN; j++) nacc += ks[j][tid] * sw2[j];
+        }
+    }
+    float* out = a.dC + ((size_t)bh * a.NCS + cc) * D * D + VW * vh;
+#pragma unroll
+    for (int x = 0; x < KPT; x++)
+        *reinterpret_cast<f32x4*>(out + (size_t)(k0 + x) * D + v0) = f32x4{acc[x][0], acc[x][1], acc[x][2], acc[x][3]};
+    if (vh == 0 && tid < D) a.Nst[((size_t)bh * a.NCS + cc) * D + tid] = nacc;
+}
+
 // gamma_c = exp(A_{e_{c-1}} - A_{e_c}), e_c the last position of chunk c (c >= 1, both chunks complete): what the state
 // at the end of chunk c - 1 decays by until the end of chunk c, and what the reverse state behind chunk c decays by
 // until it is seen from the end of chunk c - 1
@@ -387,12 +471,15 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
     const int k = idx / (D / 8), v8 = (idx % (D / 8)) * 8;
     const size_t poff = (size_t)bh * a.NG * GRAN, goff = (size_t)bh * a.NG;
     const int L = a.L;
-    const float* src = a.dC + (size_t)bh * a.NCS * D * D + (size_t)k * D + v8;
-    T* dst = reinterpret_cast<T*>(a.Cst) + (size_t)bh * a.NCS * D * D + (size_t)((k & ~15) | perm16(k & 15)) * D + v8;
+    const size_t hbase = (size_t)bh * a.NCS * D * D;
+    const float* src = a.dC + hbase + (size_t)k * D + v8;
+    const size_t koff = hbase + (size_t)state_row<T>(k) * D + v8;   // key-major: eight values of key k
     float* nst = a.Nst + (size_t)bh * a.NCS * D + tid;
     const bool vec = blockIdx.x == 0 && tid < D;
     f32x4 run0 = {0.f, 0.f, 0.f, 0.f}, run1 = {0.f, 0.f, 0.f, 0.f};
     float nrun = 0.f;
+    typedef typename Tr<T>::vec4 V4;
+    struct Pair { V4 lo, hi; };
     for (int step = 0; step < a.NCS; step++) {
         const int c = a.reverse ? a.NCS - 1 - step : step;
         const float gam = step > 0 ? carry_gamma(a, poff, goff, a.reverse ? c + 1 : c) : 0.f;
@@ -405,20 +492,30 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
             asm volatile("" : "+v"(run0[e]));
             asm volatile("" : "+v"(run1[e]));
         }
-        if (a.Cst && !a.CstT) {   // (with a value-major copy wanted, chunk_carry_t_kernel writes both layouts)
-            typedef typename Tr<T>::vec4 V4;
-            struct Pair { V4 lo, hi; };
-            Pair o;
-            if (a.Cst_lo) {   // split mode: the state as two terms
-                Pair rest;
-                Tr<T>::cvt4_split(run0, o.lo, rest.lo);
-                Tr<T>::cvt4_split(run1, o.hi, rest.hi);
-                *reinterpret_cast<Pair*>(reinterpret_cast<T*>(a.Cst_lo) + (dst - reinterpret_cast<T*>(a.Cst)) + (size_t)c * D * D) = rest;
-            } else {
-                o.lo = Tr<T>::cvt4(run0);
-                o.hi = Tr<T>::cvt4(run1);
+        Pair o, rest;
+        const bool split = a.Cst_lo || a.CstT_lo;   // split mode: the state as two terms
+        if (split) {
+            Tr<T>::cvt4_split(run0, o.lo, rest.lo);
+            Tr<T>::cvt4_split(run1, o.hi, rest.hi);
+        } else {
+            o.lo = Tr<T>::cvt4(run0);
+            o.hi = Tr<T>::cvt4(run1);
+        }
+        if (a.Cst) {
+            *reinterpret_cast<Pair*>(reinterpret_cast<T*>(a.Cst) + koff + (size_t)c * D * D) = o;
+            if (a.Cst_lo) *reinterpret_cast<Pair*>(reinterpret_cast<T*>(a.Cst_lo) + koff + (size_t)c * D * D) = rest;
+        }
+        if (a.CstT) {
+            // value-major copy, element by element (the small shapes only: at D = 128 and 256 in 16 bits
+            // chunk_carry_t_kernel turns the blocks round in LDS)
+            T* t = reinterpret_cast<T*>(a.CstT) + hbase + (size_t)c * D * D + k;
+            T* tl = a.CstT_lo ? reinterpret_cast<T*>(a.CstT_lo) + hbase + (size_t)c * D * D + k : nullptr;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const size_t r = (size_t)state_row<T>(v8 + e) * D;
+                t[r] = e < 4 ? o.lo[e & 3] : o.hi[e & 3];
+                if (tl) tl[r] = e < 4 ? rest.lo[e & 3] : rest.hi[e & 3];
             }
-            *reinterpret_cast<Pair*>(dst + (size_t)c * D * D) = o;
         }
         if (vec) {
             nrun = nrun * gam + nst[(size_t)c * D];
@@ -573,6 +670,17 @@ static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     return (int)hipGetLastError();
 }
 
+// the small shapes: plain multiply-adds for the sums, one element-wise carry for both layouts
+template <typename T, int D>
+static int launch_chunk_small(const ChunkArgs& a, hipStream_t st) {
+    if (a.precise && ((a.Cst && !a.Cst_lo) || (a.CstT && !a.CstT_lo))) return MLSTM_EINVAL;
+    if (!a.precise && (a.Cst_lo || a.CstT_lo)) return MLSTM_EINVAL;
+    if (a.dot_part) return MLSTM_EINVAL;   // (launch_anchor serves these shapes)
+    hipLaunchKernelGGL((chunk_sum_small_kernel<T, D>), dim3(a.BH * a.NCS * (D / 64)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((chunk_carry_kernel<T, D>), dim3(D * D / 8 / 256, a.BH), dim3(256), 0, st, a);
+    return (int)hipGetLastError();
+}
+
 // Sum of dD over all pairs (query behind the end of chunk c, key up to it): the forward state at that boundary
 // contracted with the reverse state, <C~_c, E_c> + n~_c . g_c.  Rounding errors of the two matrices' 16-bit entries
 // average out over the D^2 products.
@@ -583,7 +691,7 @@ __global__ __launch_bounds__(1024) void anchor_kernel(const T* __restrict__ A, c
     __shared__ float part[16];
     const int c = blockIdx.x, bh = blockIdx.y, tid = threadIdx.x;
     const size_t base = ((size_t)bh * NCS + c) * D * D;
-    typedef typename Tr<T>::frag V8;
+    typedef T V8 __attribute__((ext_vector_type(8)));
     float acc = 0.f;
     for (int e = 8 * tid; e < D * D; e += 8 * 1024) {
         f32x8 x = __builtin_convertvector(*reinterpret_cast<const V8*>(A + base + e), f32x8);
@@ -616,6 +724,9 @@ int launch_anchor(int dtype, int D, const void* A, const void* B, const void* A_
     else if (dtype == MLSTM_F16)
         hipLaunchKernelGGL(anchor_kernel<_Float16>, dim3(NCS, BH), dim3(1024), 0, st, (const _Float16*)A, (const _Float16*)B,
                            (const _Float16*)A_lo, (const _Float16*)B_lo, va, vb, anchor, D, NCS);
+    else if (dtype == MLSTM_F32)
+        hipLaunchKernelGGL(anchor_kernel<float>, dim3(NCS, BH), dim3(1024), 0, st, (const float*)A, (const float*)B, (const float*)A_lo,
+                           (const float*)B_lo, va, vb, anchor, D, NCS);
     else return MLSTM_ESHAPE;
     return (int)hipGetLastError();
 }
@@ -627,7 +738,13 @@ int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st) {
     if (dtype == MLSTM_BF16 && D == 256) return launch_chunk_t<__bf16, 256>(a, st);
     if (dtype == MLSTM_F16 && D == 128) return launch_chunk_t<_Float16, 128>(a, st);
     if (dtype == MLSTM_F16 && D == 256) return launch_chunk_t<_Float16, 256>(a, st);
+    if (dtype == MLSTM_BF16 && D == 64) return launch_chunk_small<__bf16, 64>(a, st);
+    if (dtype == MLSTM_F16 && D == 64) return launch_chunk_small<_Float16, 64>(a, st);
+    if (dtype == MLSTM_F32 && D == 64) return launch_chunk_small<float, 64>(a, st);
+    if (dtype == MLSTM_F32 && D == 128) return launch_chunk_small<float, 128>(a, st);
     return MLSTM_ESHAPE;
 }
+
+bool chunk_states_fused_dot(int dtype, int D) { return dtype != MLSTM_F32 && (D == 128 || D == 256); }
 
 }  // namespace mlstm

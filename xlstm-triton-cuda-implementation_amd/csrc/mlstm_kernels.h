@@ -231,6 +231,8 @@ struct ChunkArgs {
     float* dot_part = nullptr;
 };
 int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st);
+// whether the carry of these shapes takes ChunkArgs::dot_part (otherwise launch_anchor forms the contraction)
+bool chunk_states_fused_dot(int dtype, int D);
 
 // anchor[bh][c] = <A_c, B_c> + va_c . vb_c over two sets of states in the same layout; A_lo, B_lo (both or neither):
 // their low-order terms (split mode)
