@@ -45,3 +45,46 @@ def test_seeded_random_shapes(case):
         dtype = torch.bfloat16
     B, NH, S = r(1, 3), r(1, 4), r(1, 700)
     check(B, NH, S, D, dtype, seed=77 + case, heads=[(0, 0), (B - 1, NH - 1)])
+
+
+@pytest.mark.parametrize("D", [16, 32])
+@pytest.mark.parametrize("dtype,S", [(torch.float32, 200), (torch.float32, 1100), (torch.bfloat16, 333), (torch.float16, 1100)])
+def test_head_dimensions_below_the_smallest_tile(D, dtype, S):
+    # D = 16 and 32 (the reference's kernels take any power of two from 16 on): the wrappers pad q, k, v with zero columns
+    # to the kernels' smallest head dimension and scale q for the 1 / sqrt(D) of the scores; outputs come back at D
+    B, NH = 2, 2
+    q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=D + S, f_mean=2.0)
+    dev = [x.cuda() for x in (q, k, v, f, i, dh)]
+    h, m, b, saved = mm.mlstm_forward_save_hip(*dev[:5])
+    assert tuple(h.shape) == (B, NH, S, D) and h.dtype == dtype
+    grads = mm.mlstm_backward_saved_hip(dev[5], *dev[:5], h, m, b, saved)
+    again = mm.mlstm_backward_hip(dev[5], *dev[:5])               # recomputes the forward
+    for g_, a_ in zip(grads, again):
+        assert g_.shape == a_.shape and torch.equal(g_, a_)
+    assert tuple(grads[0].shape) == (B, NH, S, D) and tuple(grads[3].shape) == (B, NH, S)
+    sl = lambda x: x[1:2, 0:1]
+    assert_matches_oracle(dtype, *(sl(x) for x in (q, k, v, f, i, dh)), h=sl(h), m=sl(m), b=sl(b), grads=[sl(g_) for g_ in grads])
+    # through autograd, like the reference's Triton_mLSTM.apply
+    ins = [x.clone().requires_grad_(True) for x in dev[:5]]
+    mm.Triton_mLSTM.apply(*ins).backward(dev[5])
+    for x, g_ in zip(ins, grads):
+        assert torch.equal(x.grad, g_)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_sixteen_bit_head_dimension_512_runs_widened(dtype):
+    # beyond the 16-bit tile kernels' head dimensions the wrappers run the fp32 path on widened inputs: results are the
+    # fp32 results of the 16-bit inputs, rounded once to the callers' types
+    B, NH, S, D = 1, 2, 200, 512
+    q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=512, f_mean=2.0)
+    dev = [x.cuda() for x in (q, k, v, f, i, dh)]
+    ins = [x.clone().requires_grad_(True) for x in dev[:5]]
+    h = mm.Triton_mLSTM.apply(*ins)
+    h.backward(dev[5])
+    assert h.dtype == dtype and ins[0].grad.dtype == dtype and ins[3].grad.dtype == dtype
+    hr, _, _ = O.mlstm_forward_dense(q, k, v, f, i, dtype=torch.float64)
+    ref = O.mlstm_backward_dense(dh, q, k, v, f, i, dtype=torch.float64, zero_first_df=True)
+    eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11     # one rounding to the type: half an ulp, and the fp32 path's 1e-4
+    for name, got, want in zip(["h", "dq", "dk", "dv", "df", "di"], [h, *(x.grad for x in ins)], [hr, *ref]):
+        got, want = got.detach().cpu().double(), want.double()
+        assert torch.all((got - want).abs() <= eps * want.abs() + 2e-4 * float(want.abs().max())), name

@@ -480,13 +480,30 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
     float nrun = 0.f;
     typedef typename Tr<T>::vec4 V4;
     struct Pair { V4 lo, hi; };
-    for (int step = 0; step < a.NCS; step++) {
+    // The steps depend on each other through the running state only: the chunk sums, the decay factors and the vector
+    // sums of four steps are requested together (one memory round trip per four steps; with few heads this kernel is a
+    // handful of workgroups waiting for memory, step by step)
+    constexpr int AHEAD = 4;
+    for (int step0 = 0; step0 < a.NCS; step0 += AHEAD) {
+      f32x4 d0s[AHEAD], d1s[AHEAD];
+      float gams[AHEAD], nin[AHEAD];
+#pragma unroll
+      for (int u = 0; u < AHEAD; u++) {
+          const int step = step0 + u < a.NCS ? step0 + u : a.NCS - 1;
+          const int c = a.reverse ? a.NCS - 1 - step : step;
+          gams[u] = step > 0 ? carry_gamma(a, poff, goff, a.reverse ? c + 1 : c) : 0.f;
+          d0s[u] = *reinterpret_cast<const f32x4*>(src + (size_t)c * D * D);
+          d1s[u] = *reinterpret_cast<const f32x4*>(src + (size_t)c * D * D + 4);
+          nin[u] = vec ? nst[(size_t)c * D] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < AHEAD; u++) {
+        const int step = step0 + u;
+        if (step >= a.NCS) break;
         const int c = a.reverse ? a.NCS - 1 - step : step;
-        const float gam = step > 0 ? carry_gamma(a, poff, goff, a.reverse ? c + 1 : c) : 0.f;
-        const f32x4 d0 = *reinterpret_cast<const f32x4*>(src + (size_t)c * D * D);
-        const f32x4 d1 = *reinterpret_cast<const f32x4*>(src + (size_t)c * D * D + 4);
-        run0 = run0 * gam + d0;
-        run1 = run1 * gam + d1;
+        const float gam = gams[u];
+        run0 = run0 * gam + d0s[u];
+        run1 = run1 * gam + d1s[u];
 #pragma unroll
         for (int e = 0; e < 4; e++) {   // (see chunk_carry_t_kernel: the fp32 value is fixed before any conversion)
             asm volatile("" : "+v"(run0[e]));
@@ -518,9 +535,10 @@ __global__ __launch_bounds__(256) void chunk_carry_kernel(ChunkArgs a) {
             }
         }
         if (vec) {
-            nrun = nrun * gam + nst[(size_t)c * D];
+            nrun = nrun * gam + nin[u];
             nst[(size_t)c * D] = nrun;
         }
+      }
     }
 }
 

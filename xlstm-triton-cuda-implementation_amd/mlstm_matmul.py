@@ -36,6 +36,46 @@ def _check_inputs(q, k, v, f, i, precise=False):
     return B, NH, S, D, _ffi.dtype_code(q.dtype, precise), _ffi.dtype_code(f.dtype)
 
 
+# Head dimensions below the kernels' smallest tile (64) run zero-padded: the padded columns of q, k, v add nothing to a
+# score or to h, and q is scaled by sqrt(padded D / D) so that the kernels' 1 / sqrt(padded D) gives the scores their
+# 1 / sqrt(D).  The padded size is four times D: the factor is 2, exact in every type (padding 32 to 64 would round a
+# 16-bit q once more, by sqrt 2, and the row sums b would show it).
+_PADDED_D = {16: 64, 32: 128}
+
+
+def _pads(q):
+    return q.dim() == 4 and q.shape[-1] in _PADDED_D
+
+
+def _pad_last(x, Dp):
+    return None if x is None else torch.nn.functional.pad(x, (0, Dp - x.shape[-1]))
+
+
+def _pad_qkv(q, k, v):
+    D = q.shape[-1]
+    Dp = _PADDED_D[D]
+    s = (Dp / D) ** 0.5
+    return _pad_last((q.float() * s).to(q.dtype), Dp), _pad_last(k, Dp), _pad_last(v, Dp), D, s
+
+
+def _unpad_grads(grads, q, D, s):
+    dq, dk, dv, df, di = grads
+    return (dq[..., :D].float() * s).to(q.dtype), dk[..., :D].contiguous(), dv[..., :D].contiguous(), df, di
+
+
+# 16-bit tensors at head dimensions beyond the 16-bit tile kernels (512, 1024) run on the fp32 path (the scan form's
+# kernels behind the same entry points): inputs widened, outputs and gradients rounded back to the callers' types.
+_WIDENED_D = (512, 1024)
+
+
+def _widens(q):
+    return q.dim() == 4 and q.shape[-1] in _WIDENED_D and q.dtype in (torch.float16, torch.bfloat16)
+
+
+def _wide(*xs):
+    return [None if x is None else x.float().contiguous() for x in xs]
+
+
 def _dh_like(dh, h):
     """dh in h's layout (the kernels read h and dh through one set of strides)."""
     if tuple(dh.stride()) == tuple(h.stride()):
@@ -49,6 +89,13 @@ def mlstm_forward_hip(q, k, v, f, i, precise=False, gate_form="raw"):
     """Returns (h, m, b): h [B,NH,S,D] in q's dtype and dimension order in memory, m and b [B,NH,S] fp32 (reference
     mlstm_matmul.py:373-378).  gate_form: what f holds ("raw" pre-activations as in the reference, "logsigmoid", or
     "cumsum" of the log-sigmoid over the positions; fp32 gates only for the last)."""
+    if _pads(q):
+        qp, kp, vp, D, _ = _pad_qkv(q, k, v)
+        h, m, b = mlstm_forward_hip(qp, kp, vp, f, i, precise, gate_form)
+        return h[..., :D].contiguous(), m, b
+    if _widens(q):
+        h, m, b = mlstm_forward_hip(*_wide(q, k, v, f, i), False, gate_form)
+        return h.to(q.dtype), m, b
     q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
     f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
@@ -67,6 +114,15 @@ def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False,
     """Returns (dq, dk, dv, df, di) (reference mlstm_matmul.py:384-405), each in the layout of the tensor it is the
     gradient of; df is the gradient of whatever f held (gate_form).  h, m, b: the forward's outputs, or None to have
     them recomputed."""
+    if _pads(q):
+        qp, kp, vp, D, s = _pad_qkv(q, k, v)
+        have = h is not None and m is not None and b is not None
+        grads = mlstm_backward_hip(_pad_last(dh, qp.shape[-1]), qp, kp, vp, f, i, _pad_last(h, qp.shape[-1]) if have else None,
+                                   m if have else None, b if have else None, precise, gate_form)
+        return _unpad_grads(grads, q, D, s)
+    if _widens(q):   # (the fp32 path recomputes the forward it needs)
+        dq, dk, dv, df, di = mlstm_backward_hip(*_wide(dh, q, k, v, f, i), None, None, None, False, gate_form)
+        return dq.to(q.dtype), dk.to(q.dtype), dv.to(q.dtype), df.to(f.dtype), di.to(f.dtype)
     q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
     f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
@@ -96,7 +152,13 @@ def mlstm_backward_hip(dh, q, k, v, f, i, h=None, m=None, b=None, precise=False,
 
 def mlstm_forward_save_hip(q, k, v, f, i, precise=False, gate_form="raw"):
     """Forward of a training step.  Returns (h, m, b, saved): as mlstm_forward_hip, plus what the backward can reuse (the
-    states at the chunk ends of a long 16-bit sequence; None for shapes that do not run in chunks)."""
+    states at the chunk ends of a long sequence; None for shapes that do not run in chunks)."""
+    if _pads(q):
+        qp, kp, vp, D, _ = _pad_qkv(q, k, v)
+        h, m, b, saved = mlstm_forward_save_hip(qp, kp, vp, f, i, precise, gate_form)
+        return h[..., :D].contiguous(), m, b, saved
+    if _widens(q):
+        return (*mlstm_forward_hip(q, k, v, f, i, precise, gate_form), None)
     q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
     f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
@@ -116,6 +178,13 @@ def mlstm_forward_save_hip(q, k, v, f, i, precise=False, gate_form="raw"):
 
 def mlstm_backward_saved_hip(dh, q, k, v, f, i, h, m, b, saved, precise=False, gate_form="raw"):
     """Backward of a training step with the forward's outputs and its saved states (mlstm_forward_save_hip)."""
+    if _pads(q):
+        qp, kp, vp, D, s = _pad_qkv(q, k, v)
+        Dp = qp.shape[-1]
+        grads = mlstm_backward_saved_hip(_pad_last(dh, Dp), qp, kp, vp, f, i, _pad_last(h, Dp), m, b, saved, precise, gate_form)
+        return _unpad_grads(grads, q, D, s)
+    if _widens(q):
+        return mlstm_backward_hip(dh, q, k, v, f, i, None, None, None, precise, gate_form)
     q, k, v = _ffi.dense_unless_disjoint(q, k, v)   # (expanded views: see there)
     f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i, precise)
