@@ -384,6 +384,8 @@ def main():
     ap.add_argument("--precise", action="store_true", help="split mode of the 16-bit kernels (MLSTM_PRECISE)")
     ap.add_argument("--chunk-length", type=int, default=0,
                     help="measurement aid: chunk length of the 16-bit kernels (a multiple of 128; 0 = the library's choice, < 0 = no chunks)")
+    ap.add_argument("--state-kernel", type=int, default=0, choices=[0, 1, 2],
+                    help="measurement aid: 0 = the library's choice, 1 = chunk sums + carry, 2 = the one-pass kernel")
     ap.add_argument("--column-kernel", type=int, default=0, choices=[0, 1, 2, 3],
                     help="measurement aid: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -403,6 +405,7 @@ def main():
     COLUMN_KERNEL = args.column_kernel
     ffi.set_column_kernel(args.column_kernel)
     ffi.set_chunk_length(args.chunk_length)
+    ffi.set_state_kernel(args.state_kernel)
     if args.calibrate_copy:
         # 1 GiB, copied twice: four times the chip's 256 MB last-level cache, so the second copy's source comes from HBM
         # (a source that still sits in that cache reads as almost no FETCH_SIZE at all)

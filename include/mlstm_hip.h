@@ -320,6 +320,15 @@ int mlstm_set_chunk_length(int length);
  * or MLSTM_EINVAL.  No counterpart in the reference.
  */
 int mlstm_set_column_kernel(int variant);
+/*
+ * Measurement and test aid: which kernels form the chunk states of the 16-bit types at D = 128 and 256.
+ * 0 = the library's choice (chunk sums and carry today), 1 = chunk sums and carry (two kernels, any size, split mode),
+ * 2 = the one-pass kernel ((D / 64) * 2 workgroups per head walk the chunks in order, no fp32 sums through memory)
+ * wherever it can serve (not in split mode, at most 256 states per head).  The two weight different operands (V, K), so
+ * their states differ by the rounding of a weighted 16-bit operand, like two runs of different tilings.
+ * Process-wide; returns 0, or MLSTM_EINVAL.  No counterpart in the reference.
+ */
+int mlstm_set_state_kernel(int variant);
 /* The chunk length the entry points use for this shape under the current setting, 0 = the sequence is not cut
  * (measurement aid: the work a chunked kernel executes depends on it). */
 int mlstm_chunk_length_for(int S, int D, int dtype);

@@ -253,3 +253,46 @@ def test_fp32_default_chunk_length_and_many_heads():
     assert torch.equal(h1[0, 0], h[1, 2]) and torch.equal(b1[0, 0], b[1, 2])
     for name, a, w in zip(["dq", "dk", "dv", "df", "di"], g1, grads):
         assert torch.equal(a[0, 0], w[1, 2]), name
+
+
+class state_kernel:
+    def __init__(self, variant):
+        self.variant = variant
+
+    def __enter__(self):
+        ffi.set_state_kernel(self.variant)
+
+    def __exit__(self, *exc):
+        ffi.set_state_kernel(0)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("B,NH,S,D,L", [(1, 2, 1100, 256, 256), (1, 3, 1573, 128, 512), (2, 8, 2048, 256, 0), (1, 2, 1000, 128, 128), (1, 1, 4096 + 70, 128, 0)])
+def test_one_pass_state_kernel(dt, B, NH, S, D, L):
+    # the chunk states by the kernel that walks a head's chunks in order ((D / 64) * 2 workgroups per head, hand-counted
+    # direct loads): forward and backward against the oracle, and against the two-kernel form within the rounding of the
+    # weighted operand (the two weight different operands); ragged last chunks, head counts with and without the XCD order
+    dtype = DT[dt]
+    q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=S + D + L + 9, f_mean=2.0)
+    args = dev(dh, q, k, v, f, i)
+    Lc = length_in_use(L, S, D, dtype)
+    outs = []
+    for variant in (2, 1):
+        with chunk_length(L), state_kernel(variant):
+            h, m, b, saved = mm.mlstm_forward_save_hip(*args[1:])
+            got = mm.mlstm_backward_saved_hip(*args, h, m, b, saved)
+            again = mm.mlstm_backward_hip(*args, h, m, b)
+        assert ffi.lib().mlstm_kernel_error() == 0
+        for name, a, w in zip(["dq", "dk", "dv", "df", "di"], got, again):
+            assert torch.equal(a, w), name
+        outs.append([h, m, b, *got])
+    sl = lambda x: x[B - 1:B, NH - 1:NH]
+    h, m, b, *got = outs[0]
+    assert_matches_oracle(dtype, *(sl(x) for x in (q, k, v, f, i, dh)), h=sl(h), m=sl(m), b=sl(b), grads=[sl(g) for g in got], chunk_len=Lc)
+    one = rounding_noise(sl(dh), *(sl(x) for x in (q, k, v, f, i)), dtype, chunk_len=Lc)
+    sig = combined(one, one)
+    for name, x, y in zip(["h", "m", "b", "dq", "dk", "dv", "df", "di"], outs[0], outs[1]):
+        if name in ("m", "b"):
+            assert_close(sl(x), sl(y).double(), torch.float32, name + " one pass vs two kernels")
+        else:
+            assert_close(sl(x), sl(y).float(), dtype, name + " one pass vs two kernels", sig[name])

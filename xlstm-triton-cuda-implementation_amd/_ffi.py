@@ -104,6 +104,8 @@ def lib():
         L.mlstm_init.argtypes = []
         L.mlstm_set_column_kernel.restype = ci
         L.mlstm_set_column_kernel.argtypes = [ci]
+        L.mlstm_set_state_kernel.restype = ci
+        L.mlstm_set_state_kernel.argtypes = [ci]
         L.mlstm_set_spin_limit.restype = ci
         L.mlstm_set_spin_limit.argtypes = [ci]
         L.mlstm_force_generic_kernels.restype = ci
@@ -120,7 +122,8 @@ def exported_symbols():
             "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
-            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init", "mlstm_set_column_kernel"]
+            "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init", "mlstm_set_column_kernel",
+            "mlstm_set_state_kernel"]
 
 
 KERNELS = {"gates": 0, "row_fwd": 1, "col": 3, "row_dq": 4, "df": 5, "scan_state": 6, "scan_carry": 7,
@@ -135,6 +138,11 @@ def force_generic_kernels(on):
 def set_column_kernel(variant):
     """Measurement and test aid: 0 = the library's choice, 1 = col16_kernel, 2 = cold_kernel, 3 = col_kernel."""
     check_rc(lib().mlstm_set_column_kernel(int(variant)), "mlstm_set_column_kernel")
+
+
+def set_state_kernel(variant):
+    """Measurement and test aid: 0 = the library's choice, 1 = chunk sums + carry, 2 = the one-pass kernel."""
+    check_rc(lib().mlstm_set_state_kernel(int(variant)), "mlstm_set_state_kernel")
 
 
 def set_chunk_length(length):

@@ -424,6 +424,8 @@ int mlstm_chunk_length_for(int S, int D, int dtype) {
     return chunk_len_for(dtype & ~MLSTM_PRECISE, D, (size_t)S);
 }
 
+int mlstm_set_state_kernel(int variant) { return mlstm::set_state_kernel(variant); }
+
 int mlstm_set_chunk_length(int length) {
     if (length > 0 && length % 128 != 0) return MLSTM_EINVAL;
     g_chunk_override = length;
@@ -644,6 +646,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     float* gvec = c.take<float>(z.BH * w.ncs * z.D);
     float* rowinter = c.take<float>(z.BH * z.S);
     float* anchor = c.take<float>(z.BH * w.ncs * z.anchor_parts());
+    int anchor_parts = 0;
     // (the one-kernel dF pass adds the parts up; see DfArgs)
     const bool fused_anchor = w.L <= 1024 && mlstm::chunk_states_fused_dot(dtype, D);
     char* hlo_buf = c.take<char>(z.precise ? z.BH * z.S * z.D * z.el : 0);
@@ -703,7 +706,10 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
         ra2.lk = z.la; ra2.lv = z.lb;
         ra2.precise = z.precise ? 1 : 0;
         ra2.CstT_lo = z.precise ? Ev + lo_off : nullptr;
-        if (fused_anchor) { ra2.dot_with = CstT; ra2.dot_with_lo = z.precise ? CstT + lo_off : nullptr; ra2.dot_part = anchor; }
+        if (fused_anchor) {
+            ra2.dot_with = CstT; ra2.dot_with_lo = z.precise ? CstT + lo_off : nullptr; ra2.dot_part = anchor;
+            anchor_parts = mlstm::chunk_states_dot_parts(dtype, D, ra2);
+        }
         if (int e = launch_chunk_states(dtype, D, ra2, st)) return e;
         if (fused_anchor) {
         } else if (int e = launch_anchor(dtype, D, CstT, Ev, z.precise ? CstT + lo_off : nullptr, z.precise ? Ev + lo_off : nullptr, Nst, gvec, anchor,
@@ -725,7 +731,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     DfArgs da{f, colsum, rowpart, df, di, (int)z.BH, (int)z.S, (int)z.NG, (int)z.row_slices(), col_chunks ? w.L : 0, rowinter, anchor, (int)w.ncs};
     da.lg = z.lg; da.gate_form = z.gate_form; da.stamp = stamp;
     if (col_chunks && fused_anchor) {
-        da.anchor = nullptr; da.anchor_part = anchor; da.anchor_parts = (int)z.anchor_parts(); da.anchor_va = Nst; da.anchor_vb = gvec; da.D = D;
+        da.anchor = nullptr; da.anchor_part = anchor; da.anchor_parts = anchor_parts; da.anchor_va = Nst; da.anchor_vb = gvec; da.D = D;
     }
     Timed t(MLSTM_K_DF, st);
     return launch_df(gate_dtype, da, st);

@@ -652,6 +652,365 @@ __global__ __launch_bounds__(256, 4) void chunk_carry_t_kernel(ChunkArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same states in ONE pass: a workgroup owns a 64 x D/2 block of a head's state (64 keys x D/2 values) and walks the
+// head's chunks in their order (forward: first to last; reverse: last to first), the running state in its accumulators:
+// at a chunk's end the block is written in the element type (either layout, the accumulator's own rounding being the
+// only one), decays by gamma, and takes the next chunk's products.  No fp32 chunk sums travel through memory (4 + 4
+// bytes per state element in the two-kernel form above), no second launch.  (D/64) * 2 workgroups per head: for
+// launches with enough heads to fill the chip (launch_chunk_states decides); not in split mode.
+//
+// Eight waves.  Waves 4..7 bring the tiles (64 positions: K's 64 columns, V's D/2 columns, and the positions' gate
+// rows) by direct global->LDS copies, PF tiles ahead, into NS = PF + 1 stages; one tile ahead of the product they
+// leave the positions' weights in LDS and add up the vector state from K.  Waves 0..3 multiply straight out of the
+// stages -- the weights go onto the K^T fragments in registers, eight products per fragment (a weighted copy of a
+// tile in LDS costs every wave a chain of LDS round trips per tile, and those chains, not the copies or the MFMAs, set
+// the pace: measured) -- write the states and own every global store.  One barrier per tile.  The copies are counted
+// by hand: a feeder wave issues exactly NI direct loads per tile and no other vector memory operation after the
+// prologue, and waits with vmcnt((PF - 2) * NI) -- everything but the newest PF - 2 tiles -- before the barrier that
+// hands a tile on; the launch is refused if the compiled kernel uses scratch memory.
+template <typename T, int D>
+struct SeqCfg {
+    static constexpr int KR = 64, VW = D / 2;
+    static constexpr int VP = GRAN * VW * (int)sizeof(T) / 16 / 256;   // direct loads of V per feeder wave and tile
+    static constexpr int NI = 2 + VP + 1;                              // direct loads per feeder wave and tile: K, V, one gate row
+    static constexpr int MAX_STEPS = 256;                              // chunk states per head
+    static constexpr size_t K_BYTES = (size_t)GRAN * KR * sizeof(T), V_BYTES = (size_t)GRAN * VW * sizeof(T), AUX_BYTES = 4 * GRAN * sizeof(float);
+    static constexpr size_t STAGE_BYTES = K_BYTES + V_BYTES + AUX_BYTES;
+    static constexpr size_t TABLE_BYTES = MAX_STEPS * (sizeof(double) + 2 * sizeof(float));
+    static constexpr size_t RED_BYTES = 32 * KR * sizeof(float) + 64;
+    static constexpr size_t SW_BYTES = 8 * GRAN * sizeof(float);
+    // tiles requested ahead: as many stages as LDS holds
+    static constexpr int NS = (int)((160 * 1024 - TABLE_BYTES - RED_BYTES - SW_BYTES) / STAGE_BYTES) < 8
+                                  ? (int)((160 * 1024 - TABLE_BYTES - RED_BYTES - SW_BYTES) / STAGE_BYTES) : 8;
+    static constexpr int PF = NS - 1;
+    static_assert(PF >= 3 && (PF - 1) * NI < 64, "the counted wait must fit vmcnt's six bits");
+    static constexpr size_t LDS_BYTES = NS * STAGE_BYTES + SW_BYTES + TABLE_BYTES + RED_BYTES;
+    static constexpr int WPH = (D / KR) * 2;                           // workgroups per head
+};
+
+// cycle stamps of the one-pass kernel's two kinds of waves (a measurement build only: -DMLSTM_SEQ_PROF; the sums go to
+// the unused chunk-sum scratch, 16 floats per workgroup)
+#if defined(MLSTM_SEQ_PROF)
+#define SQ_DECL float prof_[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}; long long last_ = (long long)__builtin_amdgcn_s_memtime()
+#define SQ_STAMP(k) do { const long long now_ = (long long)__builtin_amdgcn_s_memtime(); prof_[k] += (float)(now_ - last_); last_ = now_; } while (0)
+#define SQ_DUMP(kind) do { if ((threadIdx.x & 255) == 0) for (int z_ = 0; z_ < 8; z_++) a.dC[(size_t)blockIdx.x * 16 + 8 * (kind) + z_] = prof_[z_]; } while (0)
+#else
+#define SQ_DECL do {} while (0)
+#define SQ_STAMP(k) do {} while (0)
+#define SQ_DUMP(kind) do {} while (0)
+#endif
+
+template <int N> __device__ __forceinline__ void dma_wait_all_but() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+template <typename T, int D, bool DOT>
+__global__ __launch_bounds__(512) void chunk_seq_kernel(ChunkArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using R = Tr<T>;
+    using Cfg = SeqCfg<T, D>;
+    typedef typename R::frag frag;
+    static_assert(R::HALF && (D == 128 || D == 256), "16-bit types, D = 128 or 256");
+    constexpr int VW = Cfg::VW, NB = VW / 64, KW = R::KW, NS = Cfg::NS, PF = Cfg::PF, NI = Cfg::NI, VP = Cfg::VP;
+    using ZK = Swz<T, 64>;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    float* const sw = reinterpret_cast<float*>(smem + NS * Cfg::STAGE_BYTES);   // [4][2][64]: the weights of two tiles, a copy per multiplying wave
+    double* const tGend = reinterpret_cast<double*>(sw + 8 * GRAN);
+    float* const tbend = reinterpret_cast<float*>(tGend + Cfg::MAX_STEPS);
+    float* const tgam = tbend + Cfg::MAX_STEPS;
+    float* const red = tgam + Cfg::MAX_STEPS;     // [32][64]: the feeders' partial vector sums of a chunk
+    float* const dotred = red + 32 * 64;          // [4]
+    auto stage_k = [&](int st) { return reinterpret_cast<T*>(smem + st * Cfg::STAGE_BYTES); };
+    auto stage_v = [&](int st) { return reinterpret_cast<T*>(smem + st * Cfg::STAGE_BYTES + Cfg::K_BYTES); };
+    auto stage_aux = [&](int st) { return reinterpret_cast<float*>(smem + st * Cfg::STAGE_BYTES + Cfg::K_BYTES + Cfg::V_BYTES); };
+
+    const bool feeder = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8) != 0;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), h = lane >> 5, c32 = lane & 31;
+    // the workgroups of a head on one XCD (they read the same K and V columns), heads dealt round the eight XCDs
+    int w, bh;
+    if ((a.BH & 7) == 0) { const int q = blockIdx.x >> 3; w = q % Cfg::WPH; bh = (blockIdx.x & 7) + 8 * (q / Cfg::WPH); }
+    else { w = blockIdx.x % Cfg::WPH; bh = blockIdx.x / Cfg::WPH; }
+    const int kq = w >> 1, vh = w & 1;
+    const int S = a.S, L = a.L, NT = L / GRAN, NCS = a.NCS;
+    const size_t poff = (size_t)bh * a.NG * GRAN, goff = (size_t)bh * a.NG;
+    const bool rev = a.reverse != 0;
+    // step s of the walk: forward chunk s (state s); reverse the positions of chunk NCS - s (state NCS - 1 - s), of which
+    // the first, the sequence's last chunk, may be short
+    const int NT0 = rev ? (S - NCS * L + GRAN - 1) / GRAN : NT;
+    const int NTOT = NT0 + (NCS - 1) * NT;
+    auto step_base = [&](int s) { return rev ? (NCS - s) * L : s * L; };
+    auto step_tiles = [&](int s) { return s == 0 ? NT0 : NT; };
+    struct Cur {   // a tile of the walk
+        int s, tt;
+    };
+    auto advance = [&](Cur& c) { if (++c.tt == step_tiles(c.s)) { c.tt = 0; c.s++; } };
+
+    // per-step tables, by everybody: reference exponent of the step's weights and the decay between steps
+    for (int s = threadIdx.x; s < NCS; s += 512) {
+        const int c = rev ? NCS - 1 - s : s;
+        const int pe = (c + 1) * L - 1;   // forward: the chunk's last position; reverse: the last position before the chunk
+        tbend[s] = a.beta2[poff + pe];
+        tGend[s] = a.G2[goff + pe / GRAN];
+        tgam[s] = s > 0 ? carry_gamma(a, poff, goff, rev ? c + 1 : c) : 0.f;
+    }
+    const float log2scale = -0.5f * __log2f((float)D);
+    const size_t rsK = (size_t)a.lk.ss, rsV = (size_t)a.lv.ss;
+    const T* Kh = reinterpret_cast<const T*>(a.K) + a.lk.head(bh) + 64 * kq;
+    const T* Vh = reinterpret_cast<const T*>(a.V) + a.lv.head(bh) + VW * vh;
+    dma_wait();        // (the last plain loads of the feeder waves: from here on their vmcnt counts direct loads only)
+    __syncthreads();
+
+    if (feeder) {
+        TileDma<T, 64, GRAN, 256> kdma;
+        TileDma<T, VW, GRAN, 256> vdma;
+        kdma.init(tid);
+        vdma.init(tid);
+        const auto krows = kdma.rows(tid, (unsigned)(rsK * sizeof(T)));
+        const auto vrows = vdma.rows(tid, (unsigned)(rsV * sizeof(T)));
+        static_assert(TileDma<T, 64, GRAN, 256>::PER_WAVE == 2 && TileDma<T, VW, GRAN, 256>::PER_WAVE == VP, "direct loads per tile");
+        // gate rows of a tile: wave 0 alpha (forward) or beta (reverse), waves 1 and 2 the dQ pass's 1/n and db (reverse; the
+        // forward repeats alpha), wave 3 the granule's G (two dwords; the other lanes read them again)
+        const float* auxsrc;
+        if (wave == 3) auxsrc = reinterpret_cast<const float*>(a.G2 + goff) + (lane & 1);
+        else if (!rev || wave == 0) auxsrc = (rev ? a.beta2 : a.alpha2) + poff + lane;
+        else auxsrc = (wave == 1 ? a.inv_n : a.db) + poff + lane;
+        const int auxstep = wave == 3 ? 2 : GRAN;   // floats per tile
+        auto issue = [&](const Cur& c, int st) __attribute__((always_inline)) {
+            const int pos0 = step_base(c.s) + GRAN * c.tt;
+            if (pos0 + GRAN <= S) {
+                kdma.issue(stage_k(st), Kh + (size_t)pos0 * rsK, krows);
+                vdma.issue(stage_v(st), Vh + (size_t)pos0 * rsV, vrows);
+            } else {   // the sequence's last tile: rows past the end are clamped (their weights are 0)
+                tile_dma<T, 64, GRAN, 256>(stage_k(st), Kh, pos0, S, tid, rsK);
+                tile_dma<T, VW, GRAN, 256>(stage_v(st), Vh, pos0, S, tid, rsV);
+            }
+            dma4(auxsrc + (size_t)(pos0 / GRAN) * auxstep, __builtin_amdgcn_readfirstlane(lds_offset_of(stage_aux(st))) + wave * 256);
+        };
+        // Tile c (landed in stage st, published by a barrier): the vector sum from K, two 16-byte pieces per thread (rows
+        // tid / 8 and tid / 8 + 32), in the workgroups that own it
+        f32x8 nacc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        const int prow = tid / ZK::CPR, pch = tid % ZK::CPR;
+        auto prepare = [&](const Cur& c, int st) __attribute__((always_inline)) {
+            if (vh != 0) return;
+            const float* ax = stage_aux(st);
+            const int pos0 = step_base(c.s) + GRAN * c.tt;
+            const float bend = tbend[c.s];
+            const float dG = (float)(rev ? *reinterpret_cast<const double*>(ax + 3 * GRAN) - tGend[c.s]
+                                         : tGend[c.s] - *reinterpret_cast<const double*>(ax + 3 * GRAN));
+            u32x4 raw[2];
+            if (vh == 0) {
+#pragma unroll
+                for (int it = 0; it < 2; it++) raw[it] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const char*>(stage_k(st)) + ZK::off(prow + 32 * it, 8 * pch));
+            }
+#pragma unroll
+            for (int it = 0; it < 2; it++) {
+                const int row = prow + 32 * it;
+                const float e = rev ? bend - ax[row] : ax[row] - bend;
+                float rho = fast_exp2(e + dG + log2scale);
+                if (pos0 + row >= S) rho = 0.f;
+                const float w2 = rev ? rho * ax[2 * GRAN + row] : rho;
+                {
+                    float x[8];
+                    unpack8<T>(raw[it], x);
+#pragma unroll
+                    for (int e8 = 0; e8 < 8; e8++) nacc[e8] += x[e8] * w2;
+                }
+            }
+            if (vh == 0 && c.tt == step_tiles(c.s) - 1) {   // the step's last tile: the partial sums go to the multiplying waves
+                *reinterpret_cast<f32x8*>(red + prow * 64 + 8 * pch) = nacc;
+#pragma unroll
+                for (int e8 = 0; e8 < 8; e8++) nacc[e8] = 0.f;
+            }
+        };
+        Cur ci{0, 0}, ct{0, 0};   // the next tile to request, the next one to prepare
+#pragma unroll
+        for (int p = 0; p < PF; p++)
+            if (p < NTOT) { issue(ci, p % NS); advance(ci); }
+        if (NTOT >= PF) dma_wait_all_but<(PF - 1) * NI>(); else dma_wait();
+        __syncthreads();   // tile 0 has landed
+        prepare(ct, 0);
+        advance(ct);
+        if (NTOT >= PF) dma_wait_all_but<(PF - 2) * NI>(); else dma_wait();
+        __syncthreads();   // tile 1 has landed
+        SQ_DECL;
+        for (int t = 0; t < NTOT; t++) {
+            if (t + PF < NTOT) { issue(ci, (t + PF) % NS); advance(ci); }
+            SQ_STAMP(0);
+            if (t + 1 < NTOT) { prepare(ct, (t + 1) % NS); advance(ct); }
+            SQ_STAMP(1);
+            if (t + PF < NTOT) dma_wait_all_but<(PF - 2) * NI>(); else dma_wait();
+            SQ_STAMP(2);
+            __syncthreads();
+            SQ_STAMP(3);
+        }
+        SQ_DUMP(0);
+    } else {
+        const int wk = wave & 1, wv = wave >> 1;
+        f32x16 acc[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int x = 0; x < 16; x++) acc[nb][x] = 0.f;
+        float nrun = 0.f;
+        Cur cm{0, 0};
+        __syncthreads();
+        __syncthreads();
+        int pending_dot = -1;   // state whose contraction's parts lie in dotred
+        // per-lane byte offsets of the transposing reads (see swz_frag_transposed), contraction step s4 = 0: K block wk and
+        // V blocks NB wv + nb; a step further lies 16 tile rows on (the swizzle key has a period of 16 rows)
+        const int tj = lane & 15, tsub = (lane >> 4) & 1;
+        int koff[2], voff[NB][2];
+#pragma unroll
+        for (int hi = 0; hi < 2; hi++) {
+            koff[hi] = ZK::off(4 * h + (tj >> 2) + 8 * hi, 32 * wk + 16 * tsub + 4 * (tj & 3));
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) voff[nb][hi] = Swz<T, VW>::off(4 * h + (tj >> 2) + 8 * hi, 32 * (NB * wv + nb) + 16 * tsub + 4 * (tj & 3));
+        }
+        auto read_tr = [&](const T* tile, const int (&off)[2], int row_bytes, int s4) __attribute__((always_inline)) {
+            const char* base = reinterpret_cast<const char*>(tile) + KW * s4 * row_bytes;
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(base + off[0]));
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(base + off[1]));
+            return __builtin_bit_cast(frag, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        };
+        float* const wt = sw + wave * 2 * GRAN;   // this wave's copies of two tiles' weights
+        // the weight of position `lane` of tile c (in stage st) into the wave's copy wb: written and read in program order
+        auto weigh = [&](const Cur& c, int st, int wb) __attribute__((always_inline)) {
+            const float* ax = stage_aux(st);
+            const int pos0 = step_base(c.s) + GRAN * c.tt;
+            const float dG = (float)(rev ? *reinterpret_cast<const double*>(ax + 3 * GRAN) - tGend[c.s]
+                                         : tGend[c.s] - *reinterpret_cast<const double*>(ax + 3 * GRAN));
+            const float e = rev ? tbend[c.s] - ax[lane] : ax[lane] - tbend[c.s];
+            float rho = fast_exp2(e + dG + log2scale);
+            if (pos0 + lane >= S) rho = 0.f;
+            wt[wb * GRAN + lane] = rev ? rho * ax[GRAN + lane] : rho;
+        };
+        constexpr int NSTEP = GRAN / KW;
+        frag af[2], bf[2][NB];
+        f32x4 w0[2], w1[2];
+        // fragment s4 of K^T holds, for the lane's key, positions 16 s4 + 4 h + (0..3) and 16 s4 + 8 + 4 h + (0..3)
+        auto rd = [&](int tile, int s4) __attribute__((always_inline)) {
+            const T* kt = stage_k(tile % NS);
+            const T* vt = stage_v(tile % NS);
+            const float* wv4 = wt + (tile & 1) * GRAN + KW * s4;
+            af[s4 & 1] = read_tr(kt, koff, ZK::ROW_BYTES, s4);
+            w0[s4 & 1] = *reinterpret_cast<const f32x4*>(wv4 + 4 * h);
+            w1[s4 & 1] = *reinterpret_cast<const f32x4*>(wv4 + 8 + 4 * h);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++) bf[s4 & 1][nb] = read_tr(vt, voff[nb], Swz<T, VW>::ROW_BYTES, s4);
+        };
+        // The reads of a tile's first step, and its weights, are requested during the tile before it (both tiles are
+        // published by then): a tile's product is a chain of LDS round trips, and with one barrier per tile nothing else
+        // would cover them.
+        Cur cn{0, 0};   // the tile whose weights are formed next
+        weigh(cn, 0, 0);
+        advance(cn);
+        rd(0, 0);
+        SQ_DECL;
+        for (int t = 0; t < NTOT; t++) {
+            if (t + 1 < NTOT) { weigh(cn, (t + 1) % NS, (t + 1) & 1); advance(cn); }
+            if (DOT && pending_dot >= 0 && tid == 0) {
+                a.dot_part[((size_t)bh * NCS + pending_dot) * Cfg::WPH + w] = (dotred[0] + dotred[1]) + (dotred[2] + dotred[3]);
+            }
+            pending_dot = -1;
+#pragma unroll
+            for (int s4 = 0; s4 < NSTEP; s4++) {
+                if (s4 + 1 < NSTEP) rd(t, s4 + 1);
+                else if (t + 1 < NTOT) rd(t + 1, 0);
+                float x[8];
+                unpack8<T>(__builtin_bit_cast(u32x4, af[s4 & 1]), x);
+                const f32x4 lo = f32x4{x[0], x[1], x[2], x[3]} * w0[s4 & 1], hi = f32x4{x[4], x[5], x[6], x[7]} * w1[s4 & 1];
+                typedef typename R::vec4 V4;
+                struct Pair { V4 lo, hi; } wa{R::cvt4(lo), R::cvt4(hi)};
+                const frag aw = __builtin_bit_cast(frag, wa);
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) R::mma(acc[nb], aw, bf[s4 & 1][nb]);
+            }
+            SQ_STAMP(0);
+            if (cm.tt == step_tiles(cm.s) - 1) {   // the step's last tile: state c leaves, the running state decays
+                const int c = rev ? NCS - 1 - cm.s : cm.s;
+                const size_t sbase = ((size_t)bh * NCS + c) * D * D;
+                float dot = 0.f;
+#pragma unroll
+                for (int nb = 0; nb < NB; nb++) {
+                    const int vg = VW * vh + 32 * (NB * wv + nb) + c32;
+                    const size_t vrow_off = sbase + (size_t)state_row<T>(vg) * D;
+#pragma unroll
+                    for (int g4 = 0; g4 < 4; g4++) {
+                        const int kg = 64 * kq + 32 * wk + 8 * g4 + 4 * h;
+                        const typename R::vec4 hi = R::cvt4(f32x4{acc[nb][4 * g4], acc[nb][4 * g4 + 1], acc[nb][4 * g4 + 2], acc[nb][4 * g4 + 3]});
+                        if (a.CstT) *reinterpret_cast<typename R::vec4*>(reinterpret_cast<T*>(a.CstT) + vrow_off + kg) = hi;
+                        if (a.Cst) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) reinterpret_cast<T*>(a.Cst)[sbase + (size_t)state_row<T>(kg + e) * D + vg] = hi[e];
+                        }
+                        if constexpr (DOT) {
+                            const f32x4 o = __builtin_convertvector(*reinterpret_cast<const typename R::vec4*>(reinterpret_cast<const T*>(a.dot_with) + vrow_off + kg), f32x4);
+                            const f32x4 x = __builtin_convertvector(hi, f32x4);
+                            dot += (x[0] * o[0] + x[1] * o[1]) + (x[2] * o[2] + x[3] * o[3]);
+                        }
+                    }
+                }
+                if constexpr (DOT) {
+                    dot = wave_scan_inclusive<OpAdd>(dot);
+                    if (lane == 63) dotred[wave] = dot;
+                    pending_dot = c;
+                }
+                if (vh == 0 && wave == 0) {   // the vector state: the feeders' partial sums of this step, carried like the matrix
+                    float sum = 0.f;
+#pragma unroll 8
+                    for (int g = 0; g < 32; g++) sum += red[g * 64 + lane];
+                    nrun = nrun * tgam[cm.s] + sum;
+                    a.Nst[((size_t)bh * NCS + c) * D + 64 * kq + lane] = nrun;
+                }
+                if (cm.s + 1 < NCS) {
+                    const float gam = tgam[cm.s + 1];
+#pragma unroll
+                    for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+                        for (int x = 0; x < 16; x++) acc[nb][x] *= gam;
+                }
+            }
+            advance(cm);
+            SQ_STAMP(1);
+            __syncthreads();
+            SQ_STAMP(3);
+        }
+        SQ_DUMP(1);
+        if (DOT && pending_dot >= 0 && tid == 0)
+            a.dot_part[((size_t)bh * NCS + pending_dot) * Cfg::WPH + w] = (dotred[0] + dotred[1]) + (dotred[2] + dotred[3]);
+    }
+#endif
+}
+
+// Whether the one-pass kernel serves a launch: on request only (set_state_kernel(2)), a table's worth of states, no split
+// mode.  Measured at B4 H8 S4096 D256 and B2 H32 S16384 D128 (256 workgroups each) it takes the same 68 / 234 us per
+// direction as the two kernels above (69 / 231 us): it moves half the bytes, but with one workgroup per CU and one
+// barrier per tile each of its waves spends 1500 to 2000 cycles per tile on some 150 instructions (cycle stamps: direct
+// loads 700, vector sum 600, products 1500, state write-out 400 per tile on average), so the launch stays with the two
+// kernels until that per-tile cost is halved (two workgroups per CU, or two tiles per barrier).
+int g_state_kernel = 0;   // 0 and 1 = chunk sums + carry, 2 = one pass where it can serve
+template <typename T, int D>
+static bool chunk_seq_serves(const ChunkArgs& a) {
+    using Cfg = SeqCfg<T, D>;
+    if (a.precise || a.NCS > Cfg::MAX_STEPS || (a.Cst && a.dot_part)) return false;
+    return g_state_kernel == 2;
+}
+template <typename T, int D>
+static int launch_chunk_seq(const ChunkArgs& a, hipStream_t st) {
+    using Cfg = SeqCfg<T, D>;
+    const dim3 grid(a.BH * Cfg::WPH);
+    if (a.dot_part) {
+        if (!a.dot_with || a.dot_with_lo) return MLSTM_EINVAL;
+        if (int rc = no_scratch_once<chunk_seq_kernel<T, D, true>>()) return rc;
+        if (hipError_t e = lds_limit_once<chunk_seq_kernel<T, D, true>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_seq_kernel<T, D, true>), grid, dim3(512), Cfg::LDS_BYTES, st, a);
+    } else {
+        if (int rc = no_scratch_once<chunk_seq_kernel<T, D, false>>()) return rc;
+        if (hipError_t e = lds_limit_once<chunk_seq_kernel<T, D, false>>(160 * 1024); e != hipSuccess) return (int)e;
+        hipLaunchKernelGGL((chunk_seq_kernel<T, D, false>), grid, dim3(512), Cfg::LDS_BYTES, st, a);
+    }
+    return (int)hipGetLastError();
+}
+
 template <typename T, int D, bool STRICT>
 static int launch_chunk_sum(const ChunkArgs& a, hipStream_t st) {
     using Cfg = ChunkCfg<T, D, STRICT>;
@@ -674,6 +1033,7 @@ static int launch_chunk_sum(const ChunkArgs& a, hipStream_t st) {
 template <typename T, int D>
 static int launch_chunk_t(const ChunkArgs& a, hipStream_t st) {
     if (a.precise && ((a.Cst && !a.Cst_lo) || (a.CstT && !a.CstT_lo))) return MLSTM_EINVAL;
+    if (chunk_seq_serves<T, D>(a)) return launch_chunk_seq<T, D>(a, st);
     if (int rc = a.precise ? launch_chunk_sum<T, D, true>(a, st) : launch_chunk_sum<T, D, false>(a, st)) return rc;
     // one carry kernel: the value-major one writes both layouts and the vector states
     if (a.dot_part && !(a.CstT && a.dot_with)) return MLSTM_EINVAL;
@@ -764,5 +1124,20 @@ int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st) {
 }
 
 bool chunk_states_fused_dot(int dtype, int D) { return dtype != MLSTM_F32 && (D == 128 || D == 256); }
+
+int chunk_states_dot_parts(int dtype, int D, const ChunkArgs& a) {
+    bool seq = false;
+    if (dtype == MLSTM_BF16 && D == 128) seq = chunk_seq_serves<__bf16, 128>(a);
+    if (dtype == MLSTM_BF16 && D == 256) seq = chunk_seq_serves<__bf16, 256>(a);
+    if (dtype == MLSTM_F16 && D == 128) seq = chunk_seq_serves<_Float16, 128>(a);
+    if (dtype == MLSTM_F16 && D == 256) seq = chunk_seq_serves<_Float16, 256>(a);
+    return seq ? (D / 64) * 2 : (D / 64) * (D / 64);
+}
+
+int set_state_kernel(int variant) {
+    if (variant < 0 || variant > 2) return MLSTM_EINVAL;
+    g_state_kernel = variant;
+    return 0;
+}
 
 }  // namespace mlstm

@@ -233,6 +233,11 @@ struct ChunkArgs {
 int launch_chunk_states(int dtype, int D, const ChunkArgs& a, hipStream_t st);
 // whether the carry of these shapes takes ChunkArgs::dot_part (otherwise launch_anchor forms the contraction)
 bool chunk_states_fused_dot(int dtype, int D);
+// partial sums per state that the launch with these arguments leaves in ChunkArgs::dot_part
+int chunk_states_dot_parts(int dtype, int D, const ChunkArgs& a);
+// test and measurement aid: 0 = the library's choice by the size of the launch, 1 = chunk sums and carry (two kernels),
+// 2 = the one-pass kernel wherever it can serve
+int set_state_kernel(int variant);
 
 // anchor[bh][c] = <A_c, B_c> + va_c . vb_c over two sets of states in the same layout; A_lo, B_lo (both or neither):
 // their low-order terms (split mode)
