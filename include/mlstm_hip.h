@@ -109,7 +109,8 @@ int mlstm_backward(const void* dH, const void* Q, const void* K, const void* V, 
  * the scan form's kernels (same function, see mlstm_scan_forward_ex): the tile kernels hold a row block's D columns
  * in accumulator registers and two D-wide tiles per stage in LDS, which ends at D = 128 in fp32 and at D = 256 in
  * 16 bits; a D = 512 16-bit variant would need the head dimension tiled as well (a second kernel family), and is not
- * built.  At those fp32 sizes the tensors must be dense, the gates fp32 pre-activations, and the backward recomputes
+ * built.  (The Python wrappers serve what lies outside these sets on the same entry points: D = 16 and 32 zero-padded to
+ * four times D with q scaled by 2, which is exact; 16-bit tensors at D = 512 / 1024 widened to fp32.)  At those fp32 sizes the tensors must be dense, the gates fp32 pre-activations, and the backward recomputes
  * the forward (h, m, b are ignored); the gated entry points and layouts of the caller's return MLSTM_ESHAPE there.
  * workspace may be NULL (the library then allocates and frees stream-ordered); otherwise it must hold
  * mlstm_workspace_bytes(MLSTM_OP_FORWARD, ...) bytes.
@@ -286,7 +287,7 @@ size_t mlstm_workspace_bytes(int op, int B, int NH, int S, int D, int dtype);
 #define MLSTM_K_SCAN_CARRY 7
 #define MLSTM_K_SCAN_OUT 8
 #define MLSTM_K_GATE_BWD 9  /* element-wise backward of the output gate (gated matmul form only) */
-#define MLSTM_K_CHUNK_STATES 10  /* chunk sums + carry of the chunked forward (16-bit, D = 128 / 256, long sequences) */
+#define MLSTM_K_CHUNK_STATES 10  /* chunk sums + carry (forward and reverse states) of sequences that run in chunks */
 #define MLSTM_K_SCAN_GLUE 11     /* row-wise and vector-sum kernels between the scans of the scan form's backward */
 int mlstm_timing_enable(int on);
 /* An event pair costs the stream about 10 us of idle time around the launch it brackets.  mlstm_timing_select narrows
@@ -305,10 +306,11 @@ int mlstm_timing_read(int kernel, double* total_ms, int* launches);
 int mlstm_force_generic_kernels(int on);
 
 /*
- * Test and measurement aid with no counterpart in the reference.  The forward of the 16-bit types at D = 128 / 256
- * cuts sequences of 1024 positions and more into chunks of 512: a row walks the keys of its own chunk and takes everything
+ * Test and measurement aid with no counterpart in the reference.  The tile kernels (every type; D = 64, 128, and 256 in
+ * 16 bits) cut sequences of 1024 positions and more into chunks -- 512 positions for the 16-bit types at D = 128 / 256,
+ * 256 at D = 64, 128 for fp32 -- : a row walks the keys of its own chunk and takes everything
  * before it from the matrix state at the end of the previous chunk (the state of mlstm_scan.py:16-26; both forms are
- * the same function).  length > 0 (a multiple of 128) forces that chunk length, length < 0 switches chunking off,
+ * the same function); the backward's keys likewise take the queries behind their chunk from a reverse state.  length > 0 (a multiple of 128) forces that chunk length, length < 0 switches chunking off,
  * 0 restores the default.  Process-wide; returns 0, or MLSTM_EINVAL for a length that is not a multiple of 128.
  * Workspace sizes depend on it: query mlstm_workspace_bytes after changing it.
  */
