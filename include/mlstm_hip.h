@@ -214,6 +214,22 @@ int mlstm_backward_gated_ex(const void* dh_gated, const void* q, const void* k, 
                             const void* i, const void* o, const void* h, const float* m, const float* b, void* dq,
                             void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S, int D, int dtype,
                             int gate_dtype, void* workspace, size_t workspace_bytes, void* stream);
+/*
+ * The two gated entry points on tensors that lie where the caller keeps them (struct mlstm_layout, as for
+ * mlstm_forward_lx / mlstm_backward_lx): q, k, v and dq, dk, dv in the qkv layout; h, h_gated, o, dh_gated and d_o in the
+ * out layout; the gates and their gradients in the gate layout.  layout == NULL: dense tensors.  The backward's written
+ * tensors must not overlap (MLSTM_EINVAL).  Not for fp32 at D >= 256 (MLSTM_ESHAPE).  No counterpart in the reference
+ * (its gate is part of mlstm_scan only).
+ */
+int mlstm_forward_gated_lx(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o,
+                           void* h, void* h_gated, float* m, float* b, int B, int NH, int S, int D, int dtype,
+                           int gate_dtype, const mlstm_layout* layout, void* workspace, size_t workspace_bytes,
+                           void* stream);
+int mlstm_backward_gated_lx(const void* dh_gated, const void* q, const void* k, const void* v, const void* f,
+                            const void* i, const void* o, const void* h, const float* m, const float* b, void* dq,
+                            void* dk, void* dv, void* df, void* di, void* d_o, int B, int NH, int S, int D, int dtype,
+                            int gate_dtype, const mlstm_layout* layout, void* workspace, size_t workspace_bytes,
+                            void* stream);
 
 /*
  * Scan-form forward with the silu(o) output gate: what mlstm_scan() launches,

@@ -212,3 +212,28 @@ def test_library_refuses_overlapping_layouts_for_tensors_it_writes():
     shared_h.out_h = 0
     assert fwd(shared_h) == -1
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dtype,B,NH,S,D", [CASES[0], CASES[1], CASES[3], CASES[4]])
+def test_gated_entry_points_in_projection_layout(dtype, B, NH, S, D):
+    # the matmul form with the output gate on [B,S,NH,D] activations: o, the gated output and its gradient travel in h's
+    # layout, and every result equals the run on dense copies bit for bit (forward, backward with the forward's outputs,
+    # backward that recomputes them, autograd)
+    from mlstm_matmul import Triton_mLSTM_gated, mlstm_backward_gated_hip, mlstm_forward_gated_hip
+    q, k, v, f, i, dh, o = (x.cuda() for x in O.make_inputs(B, NH, S, D, dtype, seed=77, with_o=True))
+    qs, ks, vs, os_, dhs, fs, is_ = bshd(q), bshd(k), bshd(v), bshd(o), bshd(dh), bsh(f), bsh(i)
+    hg0, h0, m0, b0 = mlstm_forward_gated_hip(q, k, v, f, i, o)
+    hg1, h1, m1, b1 = mlstm_forward_gated_hip(qs, ks, vs, fs, is_, os_)
+    assert torch.equal(hg0, hg1) and torch.equal(h0, h1) and torch.equal(m0, m1) and torch.equal(b0, b1)
+    assert hg1.stride() == qs.stride() and h1.stride() == qs.stride()
+    g0 = mlstm_backward_gated_hip(dh, q, k, v, f, i, o, h0, m0, b0)
+    g1 = mlstm_backward_gated_hip(dhs, qs, ks, vs, fs, is_, os_, h1, m1, b1)
+    g2 = mlstm_backward_gated_hip(dhs, qs, ks, vs, fs, is_, os_)               # recomputes h, m, b
+    for name, x0, x1, x2 in zip(list(GRAD_NAMES) + ["do"], g0, g1, g2):
+        assert torch.equal(x0, x1), name
+        assert torch.equal(x0, x2), name + " (recomputed forward)"
+    assert g1[0].stride() == qs.stride() and g1[5].stride() == qs.stride() and g1[3].stride() == fs.stride()
+    ins = [x.clone().requires_grad_(True) for x in (qs, ks, vs, fs, is_, os_)]
+    Triton_mLSTM_gated.apply(*ins).backward(dhs)
+    for name, x, g in zip(list(GRAD_NAMES) + ["do"], [ins[0], ins[1], ins[2], ins[3], ins[4], ins[5]], g0):
+        assert torch.equal(x.grad, g), name

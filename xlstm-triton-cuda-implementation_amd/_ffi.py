@@ -69,6 +69,10 @@ def lib():
         L.mlstm_forward_lx.argtypes = [vp] * 8 + [ci] * 6 + [lp, vp, sz, vp]
         L.mlstm_backward_lx.restype = ci
         L.mlstm_backward_lx.argtypes = [vp] * 14 + [ci] * 6 + [lp, vp, sz, vp]
+        L.mlstm_forward_gated_lx.restype = ci
+        L.mlstm_forward_gated_lx.argtypes = [vp] * 10 + [ci] * 6 + [lp, vp, sz, vp]
+        L.mlstm_backward_gated_lx.restype = ci
+        L.mlstm_backward_gated_lx.argtypes = [vp] * 16 + [ci] * 6 + [lp, vp, sz, vp]
         L.mlstm_forward_save_lx.restype = ci
         L.mlstm_forward_save_lx.argtypes = [vp] * 9 + [sz] + [ci] * 6 + [lp, vp, sz, vp]
         L.mlstm_backward_saved_lx.restype = ci
@@ -119,7 +123,7 @@ def lib():
 def exported_symbols():
     return ["mlstm_forward", "mlstm_backward", "mlstm_forward_ex", "mlstm_forward_noalloc_ex", "mlstm_backward_ex", "mlstm_scan_forward_ex",
             "mlstm_scan_backward_ex", "mlstm_scan_forward_save_ex", "mlstm_scan_backward_saved_ex", "slstm_saved_bytes", "slstm_workspace_bytes", "slstm_forward_ex", "slstm_backward_ex", "mlstm_forward_lx", "mlstm_backward_lx", "mlstm_forward_save_lx", "mlstm_backward_saved_lx",
-            "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
+            "mlstm_forward_gated_ex", "mlstm_backward_gated_ex", "mlstm_forward_gated_lx", "mlstm_backward_gated_lx", "mlstm_set_chunk_length", "mlstm_chunk_length_for",
             "mlstm_saved_state_bytes", "mlstm_forward_save_ex", "mlstm_backward_saved_ex",
             "mlstm_workspace_bytes", "mlstm_version", "mlstm_timing_enable", "mlstm_timing_select", "mlstm_timing_read",
             "mlstm_force_generic_kernels", "mlstm_kernel_error", "mlstm_set_spin_limit", "mlstm_init", "mlstm_set_column_kernel",

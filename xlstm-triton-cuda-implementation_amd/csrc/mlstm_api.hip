@@ -584,13 +584,21 @@ int mlstm_forward_save_lx(const void* q, const void* k, const void* v, const voi
 int mlstm_forward_gated_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
                            void* h_gated, float* m, float* b, int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace,
                            size_t workspace_bytes, void* stream) {
+    return mlstm_forward_gated_lx(q, k, v, f, i, o, h, h_gated, m, b, B, NH, S, D, dtype, gate_dtype, nullptr, workspace, workspace_bytes, stream);
+}
+
+int mlstm_forward_gated_lx(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
+                           void* h_gated, float* m, float* b, int B, int NH, int S, int D, int dtype, int gate_dtype,
+                           const mlstm_layout* layout, void* workspace, size_t workspace_bytes, void* stream) {
     if (!q || !k || !v || !f || !i || !o || !h || !h_gated || B <= 0 || NH <= 0 || S <= 0 || !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
     const int dtype_arg = dtype;
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (layout && z.scan_engine()) return MLSTM_ESHAPE;
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {q, k, v, o, h, h_gated}, false, true, false)) return rc;   // (o, h, h_gated: the layout of h)
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.fwd(), st)) return rc;
     return forward_impl(q, k, v, f, i, h, m, b, z, D, dtype, gate_dtype, (char*)sc.p, st, nullptr, nullptr, nullptr, nullptr, nullptr,
@@ -604,7 +612,7 @@ namespace {
 // the backward on a workspace of Sizes::bwd() bytes; arguments already validated
 int backward_impl(const void* dh, const void* q, const void* k, const void* v, const void* f, const void* i, const void* h, const float* m,
                   const float* b, void* dq, void* dk, void* dv, void* df, void* di, const Sizes& z, int D, int dtype, int gate_dtype,
-                  char* ws, hipStream_t st, const char* saved = nullptr) {
+                  char* ws, hipStream_t st, const char* saved = nullptr, const Lay* h_layout = nullptr) {
     if (z.scan_engine()) {   // (recomputes the forward it needs; h, m, b are not read)
         if (!is_dense(z.la, (long long)z.S, (long long)z.D) || !is_dense(z.lb, (long long)z.S, (long long)z.D) ||
             !is_dense(z.lg, (long long)z.S, 1) || z.gate_form != MLSTM_GATE_RAW || gate_dtype != MLSTM_F32)
@@ -657,7 +665,7 @@ int backward_impl(const void* dh, const void* q, const void* k, const void* v, c
     // Split mode needs h beyond the element type's precision for dh . h: either the forward left the low-order part
     // (saved), or the forward is run again here
     const bool have_fwd = h && m && b && (!z.precise || h_lo);
-    Lay lh = z.lb;   // layout of the forward output the dQ pass reads
+    Lay lh = h_layout ? *h_layout : z.lb;   // layout of the forward output the dQ pass reads (dh's, unless the caller says otherwise)
     if (have_fwd) {
         // gates only: alpha, beta, G (and m again, into the workspace) are cheap to rebuild; so are the chunk states
         G2 = w.G2; alpha2 = w.alpha2; beta2 = w.beta2; ek2 = w.ek2; amax2 = w.amax2; mm = w.mw;
@@ -796,6 +804,14 @@ int mlstm_backward_saved_lx(const void* dh, const void* q, const void* k, const 
 int mlstm_backward_gated_ex(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i, const void* o,
                             const void* h, const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, void* d_o,
                             int B, int NH, int S, int D, int dtype, int gate_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+    return mlstm_backward_gated_lx(dh_gated, q, k, v, f, i, o, h, m, b, dq, dk, dv, df, di, d_o, B, NH, S, D, dtype, gate_dtype, nullptr, workspace,
+                                   workspace_bytes, stream);
+}
+
+int mlstm_backward_gated_lx(const void* dh_gated, const void* q, const void* k, const void* v, const void* f, const void* i, const void* o,
+                            const void* h, const float* m, const float* b, void* dq, void* dk, void* dv, void* df, void* di, void* d_o,
+                            int B, int NH, int S, int D, int dtype, int gate_dtype, const mlstm_layout* layout, void* workspace,
+                            size_t workspace_bytes, void* stream) {
     if (!dh_gated || !q || !k || !v || !f || !i || !o || !dq || !dk || !dv || !df || !di || !d_o || B <= 0 || NH <= 0 || S <= 0 ||
         !good_dtype_arg(dtype) || !good_dtype(gate_dtype))
         return MLSTM_EINVAL;
@@ -803,7 +819,10 @@ int mlstm_backward_gated_ex(const void* dh_gated, const void* q, const void* k, 
     dtype &= ~MLSTM_PRECISE;
     if (!good_shape(D, dtype) || S > 131072) return MLSTM_ESHAPE;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    Sizes z = sizes_of(B, NH, S, D, dtype_arg);
+    if (layout && z.scan_engine()) return MLSTM_ESHAPE;
+    // dh_gated, o, h and d_o in the layout of h; q, k, v and their gradients, the gates and theirs as in mlstm_backward_lx
+    if (int rc = apply_layout(z, layout, NH, gate_dtype, {dh_gated, q, k, v, o, h, dq, dk, dv, d_o}, true, true, true)) return rc;
     Scratch sc;
     if (int rc = sc.get(workspace, workspace_bytes, z.bwd_gated(), st)) return rc;
     char* ws = (char*)sc.p;
@@ -812,15 +831,27 @@ int mlstm_backward_gated_ex(const void* dh_gated, const void* q, const void* k, 
     char* hown = c.take<char>(z.BH * z.S * z.D * z.el);
     float* mown = c.take<float>(z.BH * z.S);
     float* bown = c.take<float>(z.BH * z.S);
-    if (!(h && m && b)) {  // the ungated h is an input of the gate's own backward: rebuild it (and m, b) first
-        if (int rc = forward_impl(q, k, v, f, i, hown, mown, bown, z, D, dtype, gate_dtype, ws, st)) return rc;
+    const Lay dense = dense_layout(NH, (long long)z.S, (long long)z.D);
+    Lay lh = z.lb;
+    if (!(h && m && b)) {  // the ungated h is an input of the gate's own backward: rebuild it (and m, b) first, dense
+        Sizes zf = z;
+        zf.lb = dense;
+        if (int rc = forward_impl(q, k, v, f, i, hown, mown, bown, zf, D, dtype, gate_dtype, ws, st)) return rc;
         h = hown; m = mown; b = bown;
+        lh = dense;
     }
     {
         Timed t(MLSTM_K_GATE_BWD, st);
-        if (int rc = launch_gate_backward(dtype, dh_gated, o, h, dh, d_o, z.BH * z.S * z.D, st)) return rc;
+        if (!layout) {
+            if (int rc = launch_gate_backward(dtype, dh_gated, o, h, dh, d_o, z.BH * z.S * z.D, st)) return rc;
+        } else if (int rc = launch_gate_backward_rows(dtype, dh_gated, o, h, dh, d_o, (int)z.BH, (int)z.S, (int)z.D, z.lb, lh, dense, st)) {
+            return rc;
+        }
     }
-    return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, z, D, dtype, gate_dtype, ws, st);
+    // the ungated upstream gradient is the library's own, dense; h stays where it is
+    Sizes zb = z;
+    zb.lb = dense;
+    return backward_impl(dh, q, k, v, f, i, h, m, b, dq, dk, dv, df, di, zb, D, dtype, gate_dtype, ws, st, nullptr, &lh);
 }
 
 int mlstm_forward(const void* Q, const void* K, const void* V, const void* F, const void* I, void* H, unsigned S) {

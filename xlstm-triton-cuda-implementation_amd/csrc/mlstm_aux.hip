@@ -220,6 +220,58 @@ __global__ __launch_bounds__(256) void gate_backward_kernel(const T* __restrict_
     }
 }
 
+// The same over [BH, S, D] tensors that lie where the caller keeps them: dh_out, o and d_o in layout lx, h in layout lh, dh
+// (the library's own) in layout ld; rows of D contiguous elements, 16 bytes per lane.
+template <typename T>
+__global__ __launch_bounds__(256) void gate_backward_rows_kernel(const T* __restrict__ dh_out, const T* __restrict__ o, const T* __restrict__ h,
+                                                                 T* __restrict__ dh, T* __restrict__ d_o, int S, int D, size_t nvec, Lay lx,
+                                                                 Lay lh, Lay ld) {
+    constexpr int EPV = 16 / (int)sizeof(T);
+    typedef T Vec __attribute__((ext_vector_type(EPV)));
+    typedef float FVec __attribute__((ext_vector_type(EPV)));
+    const int vpr = D / EPV;   // vectors per row
+    for (size_t v = (size_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (size_t)gridDim.x * 256) {
+        const size_t row = v / vpr;
+        const int c = (int)(v % vpr) * EPV, bh = (int)(row / S), s = (int)(row % S);
+        const size_t ox = lx.head(bh) + (size_t)s * lx.ss + c, oh = lh.head(bh) + (size_t)s * lh.ss + c, od = ld.head(bh) + (size_t)s * ld.ss + c;
+        const FVec g = __builtin_convertvector(*reinterpret_cast<const Vec*>(dh_out + ox), FVec);
+        const FVec ov = __builtin_convertvector(*reinterpret_cast<const Vec*>(o + ox), FVec);
+        const FVec hv = __builtin_convertvector(*reinterpret_cast<const Vec*>(h + oh), FVec);
+        FVec a, b;
+#pragma unroll
+        for (int e = 0; e < EPV; e++) {
+            const float sg = 1.0f / (1.0f + __expf(-ov[e]));
+            a[e] = g[e] * ov[e] * sg;
+            b[e] = g[e] * hv[e] * sg * (1.0f + ov[e] * (1.0f - sg));
+        }
+        *reinterpret_cast<Vec*>(dh + od) = __builtin_convertvector(a, Vec);
+        *reinterpret_cast<Vec*>(d_o + ox) = __builtin_convertvector(b, Vec);
+    }
+}
+
+template <typename T>
+static int launch_gate_backward_rows_t(const void* dh_out, const void* o, const void* h, void* dh, void* d_o, int BH, int S, int D,
+                                       const Lay& lx, const Lay& lh, const Lay& ld, hipStream_t st) {
+    const size_t nvec = (size_t)BH * S * D / (16 / sizeof(T));
+    const size_t want = (nvec + 255) / 256;
+    const unsigned blocks = (unsigned)(want < 256 * 16 ? (want ? want : 1) : 256 * 16);
+    hipLaunchKernelGGL(gate_backward_rows_kernel<T>, dim3(blocks), dim3(256), 0, st, reinterpret_cast<const T*>(dh_out),
+                       reinterpret_cast<const T*>(o), reinterpret_cast<const T*>(h), reinterpret_cast<T*>(dh), reinterpret_cast<T*>(d_o), S, D,
+                       nvec, lx, lh, ld);
+    return (int)hipGetLastError();
+}
+
+int launch_gate_backward_rows(int dtype, const void* dh_out, const void* o, const void* h, void* dh, void* d_o, int BH, int S, int D,
+                              const Lay& lx, const Lay& lh, const Lay& ld, hipStream_t st) {
+    if (D % 8) return MLSTM_EINVAL;
+    switch (dtype) {
+        case MLSTM_F32: return launch_gate_backward_rows_t<float>(dh_out, o, h, dh, d_o, BH, S, D, lx, lh, ld, st);
+        case MLSTM_F16: return launch_gate_backward_rows_t<_Float16>(dh_out, o, h, dh, d_o, BH, S, D, lx, lh, ld, st);
+        case MLSTM_BF16: return launch_gate_backward_rows_t<__bf16>(dh_out, o, h, dh, d_o, BH, S, D, lx, lh, ld, st);
+    }
+    return MLSTM_EINVAL;
+}
+
 template <typename T>
 static int launch_gate_backward_t(const void* dh_out, const void* o, const void* h, void* dh, void* d_o, size_t n, hipStream_t st) {
     const size_t nvec = n / (16 / sizeof(T));

@@ -247,6 +247,9 @@ int launch_anchor(int dtype, int D, const void* A, const void* B, const void* A_
 // Backward of the output gate h_out = silu(o) * h, element-wise over n elements (n a multiple of 8):
 //   dh = dh_out * silu(o)   (the upstream gradient of the ungated form),   d_o = dh_out * h * silu'(o).
 int launch_gate_backward(int dtype, const void* dh_out, const void* o, const void* h, void* dh, void* d_o, size_t n, hipStream_t st);
+// the same over [BH, S, D] tensors in layouts: dh_out, o, d_o in lx, h in lh, dh in ld
+int launch_gate_backward_rows(int dtype, const void* dh_out, const void* o, const void* h, void* dh, void* d_o, int BH, int S, int D,
+                              const Lay& lx, const Lay& lh, const Lay& ld, hipStream_t st);
 
 struct ScanArgs {
     const float* q; const float* k; const float* v; const float* o;

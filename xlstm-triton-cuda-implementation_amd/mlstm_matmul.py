@@ -10,7 +10,8 @@ Beyond the reference: q, k, v need not be contiguous [B,NH,S,D].  Any [B,NH,S,D]
 contiguous is taken as it is (``x.view(B, S, NH, D).transpose(1, 2)`` of a projection's output, or the three slices of
 a fused q/k/v projection), h comes back in the same dimension order and every gradient in the layout of its tensor;
 ``gate_form`` lets f arrive as its log-sigmoid or as the cumulative sum of that (the step the reference's
-cutlass-src-hopper/mlstm_forward.cu:201 suggests fusing into the projection).  The gated variants take dense tensors.
+cutlass-src-hopper/mlstm_forward.cu:201 suggests fusing into the projection).  The gated variants take the same views
+(o, the gated output and its gradient in h's layout).
 """
 import torch
 
@@ -266,45 +267,57 @@ class Triton_mLSTM_precise(torch.autograd.Function):
 # Triton_mLSTM_gated gives that function a backward.
 # ---------------------------------------------------------------------------------------------------------------
 def mlstm_forward_gated_hip(q, k, v, f, i, o):
-    """Returns (h_gated, h, m, b); h is the ungated output, which the backward needs."""
+    """Returns (h_gated, h, m, b); h is the ungated output, which the backward needs.  q, k, v in one layout (as for
+    mlstm_forward_hip); o is taken in the layout h is written in (q's dimension order, dense), or copied into it."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
-    for name, t in (("q", q), ("k", k), ("v", v), ("f", f), ("i", i)):
-        _ffi.require(t, name)   # the gated entry points take dense tensors
-    _ffi.require(o, "o", q.shape)
+    if not o.is_cuda or tuple(o.shape) != tuple(q.shape):
+        raise ValueError(f"o must be a GPU tensor of q's shape, got {tuple(o.shape)} on {o.device}")
     if o.dtype != q.dtype:
         raise TypeError("o must have q's dtype")
-    h, hg = torch.empty_like(q), torch.empty_like(q)
+    h = _ffi.dense_in_order_of(q)
+    hg = _ffi.strided_like(h)[0]
+    o = _dh_like(o, h)
     m = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
     b = torch.empty((B, NH, S), device=q.device, dtype=torch.float32)
+    lay = _ffi.layout(q, h, f)
     ws, n = _ffi.workspace(_ffi.OP_FORWARD_GATED, B, NH, S, D, dt, q.device)
-    rc = _ffi.lib().mlstm_forward_gated_ex(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o), _ffi.ptr(h),
-                                           _ffi.ptr(hg), _ffi.ptr(m), _ffi.ptr(b), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n,
+    rc = _ffi.lib().mlstm_forward_gated_lx(_ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o), _ffi.ptr(h),
+                                           _ffi.ptr(hg), _ffi.ptr(m), _ffi.ptr(b), B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n,
                                            _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_forward_gated_ex")
+    _ffi.check_rc(rc, "mlstm_forward_gated_lx")
     return hg, h, m, b
 
 
 def mlstm_backward_gated_hip(dhg, q, k, v, f, i, o, h=None, m=None, b=None):
-    """Returns (dq, dk, dv, df, di, do) for the gradient dhg of the gated output."""
+    """Returns (dq, dk, dv, df, di, do) for the gradient dhg of the gated output, each in the layout of its tensor (do in
+    the layout the kernels read o in: h's when h is given, else q's dimension order, dense)."""
+    q, k, v = _ffi.dense_unless_disjoint(q, k, v)
+    f, i = _ffi.dense_unless_disjoint(f, i)
     B, NH, S, D, dt, gdt = _check_inputs(q, k, v, f, i)
-    for name, t in (("q", q), ("k", k), ("v", v), ("f", f), ("i", i)):
-        _ffi.require(t, name)   # the gated entry points take dense tensors
-    _ffi.require(o, "o", q.shape)
-    _ffi.require(dhg, "dh", q.shape)
+    for name, t in (("o", o), ("dh", dhg)):
+        if not t.is_cuda or tuple(t.shape) != tuple(q.shape):
+            raise ValueError(f"{name} must be a GPU tensor of q's shape, got {tuple(t.shape)} on {t.device}")
     if dhg.dtype != q.dtype or o.dtype != q.dtype:
         raise TypeError("dh and o must have q's dtype")
-    dq, dk, dv, do = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(o)
-    df, di = torch.empty_like(f), torch.empty_like(i)
-    ws, n = _ffi.workspace(_ffi.OP_BACKWARD_GATED, B, NH, S, D, dt, q.device)
     if h is None or m is None or b is None:
         h = m = b = None
+        like = _ffi.dense_in_order_of(q)
     else:
-        _ffi.require(h, "h", q.shape)
-    rc = _ffi.lib().mlstm_backward_gated_ex(_ffi.ptr(dhg), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o),
+        _ffi.require_rows(h, "h", q.shape)
+        like = h
+    o, dhg = _dh_like(o, like), _dh_like(dhg, like)
+    dq, dk, dv = _ffi.strided_like(q, 3)
+    do = _ffi.strided_like(like)[0]
+    df, di = _ffi.strided_like(f, 2)
+    lay = _ffi.layout(q, like, f)
+    ws, n = _ffi.workspace(_ffi.OP_BACKWARD_GATED, B, NH, S, D, dt, q.device)
+    rc = _ffi.lib().mlstm_backward_gated_lx(_ffi.ptr(dhg), _ffi.ptr(q), _ffi.ptr(k), _ffi.ptr(v), _ffi.ptr(f), _ffi.ptr(i), _ffi.ptr(o),
                                             _ffi.ptr(h), _ffi.ptr(m), _ffi.ptr(b), _ffi.ptr(dq), _ffi.ptr(dk), _ffi.ptr(dv),
-                                            _ffi.ptr(df), _ffi.ptr(di), _ffi.ptr(do), B, NH, S, D, dt, gdt, _ffi.ptr(ws), n,
+                                            _ffi.ptr(df), _ffi.ptr(di), _ffi.ptr(do), B, NH, S, D, dt, gdt, lay, _ffi.ptr(ws), n,
                                             _ffi.stream_ptr())
-    _ffi.check_rc(rc, "mlstm_backward_gated_ex")
+    _ffi.check_rc(rc, "mlstm_backward_gated_lx")
     return dq, dk, dv, df, di, do
 
 
@@ -325,7 +338,7 @@ class Triton_mLSTM_gated(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dhg):
-        assert dhg.is_contiguous()
+        assert dhg.stride(-1) == 1 or dhg.shape[-1] == 1, "dh must have a contiguous head dimension"
         q, k, v, f, i, o, m, b, h = ctx.saved_tensors
         dq, dk, dv, df, di, do = mlstm_backward_gated_hip(dhg, q, k, v, f, i, o, h, m, b)
         return dq, dk, dv, df, di, do, None, None
