@@ -237,3 +237,20 @@ def test_gated_entry_points_in_projection_layout(dtype, B, NH, S, D):
     Triton_mLSTM_gated.apply(*ins).backward(dhs)
     for name, x, g in zip(list(GRAD_NAMES) + ["do"], [ins[0], ins[1], ins[2], ins[3], ins[4], ins[5]], g0):
         assert torch.equal(x.grad, g), name
+
+
+def test_scan_form_takes_views_through_one_copy():
+    # the scan kernels are dense; the wrapper copies views once, so a [B,S,NH,D] view gives the dense run's bits
+    from mlstm_scan import mlstm_scan
+    B, NH, S, D = 2, 2, 200, 128
+    q, k, v, f, i, dh, o = (x.cuda() for x in O.make_inputs(B, NH, S, D, torch.float32, seed=5, with_o=True))
+    dense = [x.clone().requires_grad_(True) for x in (q, k, v, f, i, o)]
+    views = [x.clone().requires_grad_(True) for x in (bshd(q), bshd(k), bshd(v), bsh(f), bsh(i), bshd(o))]
+    assert not views[0].is_contiguous()
+    h0 = mlstm_scan(*dense)
+    h1 = mlstm_scan(*views)
+    assert torch.equal(h0, h1)
+    h0.backward(dh)
+    h1.backward(bshd(dh))
+    for a, b_ in zip(dense, views):
+        assert torch.equal(a.grad, b_.grad)

@@ -30,7 +30,14 @@ def _check(q, k, v, f, i, o):
     return B, NH, S, D
 
 
+def _dense(*ts):
+    """The scan kernels take dense [B,NH,S,D] / [B,NH,S] tensors: views in another layout ([B,S,NH,D] activations, slices
+    of a fused projection) are copied once, here (the matmul form's entry points address such views in place instead)."""
+    return [t if (t is None or t.is_contiguous()) else t.contiguous() for t in ts]
+
+
 def mlstm_scan_forward_hip(q, k, v, f, i, o):
+    q, k, v, f, i, o = _dense(q, k, v, f, i, o)
     B, NH, S, D = _check(q, k, v, f, i, o)
     h = torch.empty_like(q)
     ws, n = _ffi.workspace(_ffi.OP_SCAN_FORWARD, B, NH, S, D, _ffi.F32, q.device)
@@ -43,6 +50,7 @@ def mlstm_scan_forward_hip(q, k, v, f, i, o):
 def mlstm_scan_forward_save_hip(q, k, v, f, i, o):
     """The forward of a training step: (h, h_ungated, b), the last two (the output before silu(o), the normaliser sums) kept
     for ``mlstm_scan_backward_hip`` so that it does not form them again."""
+    q, k, v, f, i, o = _dense(q, k, v, f, i, o)
     B, NH, S, D = _check(q, k, v, f, i, o)
     h, h_ungated = torch.empty_like(q), torch.empty_like(q)
     b = torch.empty((B, NH, S), dtype=torch.float32, device=q.device)
@@ -58,6 +66,7 @@ def mlstm_scan_backward_hip(dh, q, k, v, f, i, o, h_ungated=None, b=None):
     """Gradients (dq, dk, dv, df, di, do) of ``mlstm_scan`` for the output gradient ``dh``; df[..., 0] = 0 as in
     mlstm_matmul.py:320-333.  Nothing but the inputs is needed: the forward is run again inside, unless ``h_ungated`` and
     ``b`` of ``mlstm_scan_forward_save_hip`` are handed over (the same bits either way)."""
+    dh, q, k, v, f, i, o, h_ungated, b = _dense(dh, q, k, v, f, i, o, h_ungated, b)
     B, NH, S, D = _check(q, k, v, f, i, o)
     _ffi.require(dh, "dh", q.shape)
     if dh.dtype != torch.float32:
@@ -91,7 +100,7 @@ class Scan_mLSTM(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dh):
-        return mlstm_scan_backward_hip(dh.contiguous(), *ctx.saved_tensors)
+        return mlstm_scan_backward_hip(dh, *ctx.saved_tensors)
 
 
 def mlstm_scan(q, k, v, f, i, o, reduce_block_size=4, value_block_size=4, num_warps=8):
