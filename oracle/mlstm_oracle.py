@@ -298,7 +298,8 @@ def mlstm_rounding_noise(dh, q, k, v, f, i, dtype, work_dtype=torch.float64, chu
     q_i dh_i^T / sqrt(D), both stored in ``dtype``: every output gains the rounding of the state it is contracted
     with, and the row and column sums of dD of those far pairs, now q_i . dQ_i and k_j . dK_j, gain a per-position
     error that the running sum of df accumulates between the chunk boundaries, where it is pinned to sum <C~, E>
-    (a bridge: what a chunk's own sum misses of the next pinned value is spread evenly over the chunk).
+    (a bridge: what a chunk's own sum misses of the next pinned value is spread evenly over the chunk); the pinned
+    values carry the rounding of the two states' entries, which averages out over the D^2 products but not to nothing.
 
     Returns a tuple of tensors shaped like the outputs, in ``work_dtype`` (float32 halves the memory of the S x S
     intermediates of very long sequences)."""
@@ -329,6 +330,7 @@ def mlstm_rounding_noise(dh, q, k, v, f, i, dtype, work_dtype=torch.float64, chu
             var_dk = u2 * ((G ** 2).T @ (Q ** 2))
             var_dv = u2 * ((W ** 2).T @ (dH ** 2))
             var_x = torch.zeros(S, dtype=work_dtype)     # per-position error of (column sum - row sum) of dD, far pairs
+            var_anchor = torch.zeros(max(ncs, 1), dtype=work_dtype)   # of the pinned running sums sqrt(D) <C~_c, E_c>
             if ncs > 0:
                 pos = torch.arange(S)
                 cidx = torch.clamp(pos // L, max=ncs)
@@ -343,6 +345,9 @@ def mlstm_rounding_noise(dh, q, k, v, f, i, dtype, work_dtype=torch.float64, chu
                     Cst = (K * (sc * dp[e])[:, None]).T @ V                                         # [key index, value index]
                     rho = torch.where(pos > e, dp[:, e] / dp[e, e], torch.zeros((), dtype=work_dtype))
                     Est = (Q * (sc * rho / n)[:, None]).T @ dH
+                    # both states enter the contraction rounded, every entry on its own: the products' errors add up in
+                    # quadrature (they average out over the D^2 entries, but not to nothing)
+                    var_anchor[c] = 2.0 * u2 * ((Cst * Est) ** 2).sum() / (sc * sc)
                     dec2 = ((dp[rows, e] / dp[e, e]) / n[rows]) ** 2
                     w2 = dp[e, keys] ** 2
                     var_h[rows] += u2 * ((Q[rows] ** 2) @ (Cst ** 2)) * (dp[rows, e] / dp[e, e] / n[rows])[:, None] ** 2
@@ -367,11 +372,12 @@ def mlstm_rounding_noise(dh, q, k, v, f, i, dtype, work_dtype=torch.float64, chu
                     lo, hi = c * L, min((c + 1) * L, S) if c < ncs else S
                     vx = var_x[lo:hi]
                     P = torch.cumsum(vx, 0) - vx                                # sum over positions before tau
+                    va0 = var_anchor[c - 1] if c > 0 else torch.zeros((), dtype=work_dtype)   # the pinned value the chunk starts from
                     if c < ncs:
                         tau = torch.arange(hi - lo, dtype=work_dtype) / float(L)
-                        var_run[lo:hi] += (1 - tau) ** 2 * P + tau ** 2 * (vx.sum() - P)
+                        var_run[lo:hi] += (1 - tau) ** 2 * (P + va0) + tau ** 2 * (vx.sum() - P + var_anchor[c])
                     else:
-                        var_run[lo:hi] += P
+                        var_run[lo:hi] += P + va0
             var_df = torch.sigmoid(-f[bi, hi_]) ** 2 * var_run
             for o_, val in zip(outs, (var_h, var_dq, var_dk, var_dv, var_df, var_di)):
                 o_[bi, hi_] = val.clamp_min(0).sqrt()

@@ -88,3 +88,43 @@ def test_sixteen_bit_head_dimension_512_runs_widened(dtype):
     for name, got, want in zip(["h", "dq", "dk", "dv", "df", "di"], [h, *(x.grad for x in ins)], [hr, *ref]):
         got, want = got.detach().cpu().double(), want.double()
         assert torch.all((got - want).abs() <= eps * want.abs() + 2e-4 * float(want.abs().max())), name
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_seeded_random_long_shapes_and_kernel_switches(case):
+    # lengths on both sides of the chunking threshold, every type, forced chunk lengths, split mode, each column kernel and
+    # both state-kernel forms, three forget-gate regimes: forward + backward (with the forward's saved states, and
+    # recomputing them: the same bits) against the oracle under the rule of the arithmetic in use
+    import random
+    from _mlstm_pkg import submodule
+    ffi = submodule("_ffi")
+    rng = random.Random(9000 + case)
+    dtype = [torch.float32, torch.float16, torch.bfloat16][case % 3]
+    D = rng.choice([64, 128] if dtype == torch.float32 else [64, 128, 256])
+    B, NH = rng.randint(1, 2), rng.randint(1, 3)
+    S = rng.choice([rng.randint(900, 1400), rng.randint(1024, 2600)])
+    L = rng.choice([0, 0, 128, 256, 384, -1])
+    precise = dtype != torch.float32 and rng.random() < 0.3
+    colk, statek = rng.choice([0, 0, 1, 2, 3]), rng.choice([0, 2])
+    fmean = rng.choice([0.0, 2.0, 4.0])
+    q, k, v, f, i, dh = O.make_inputs(B, NH, S, D, dtype, seed=9000 + case, f_mean=fmean)
+    dev = [x.cuda() for x in (dh, q, k, v, f, i)]
+    try:
+        ffi.set_chunk_length(L)
+        ffi.set_column_kernel(colk)
+        ffi.set_state_kernel(statek)
+        h, m, b, saved = mm.mlstm_forward_save_hip(*dev[1:], precise=precise)
+        grads = mm.mlstm_backward_saved_hip(*dev, h, m, b, saved, precise=precise)
+        again = mm.mlstm_backward_hip(*dev, precise=precise)
+        torch.cuda.synchronize()
+        assert ffi.lib().mlstm_kernel_error() == 0
+        Lc = int(ffi.lib().mlstm_chunk_length_for(S, D, ffi.dtype_code(dtype)))
+    finally:
+        ffi.set_chunk_length(0)
+        ffi.set_column_kernel(0)
+        ffi.set_state_kernel(0)
+    for name, x, y in zip(["dq", "dk", "dv", "df", "di"], grads, again):
+        assert torch.equal(x, y), name
+    sl = lambda x: x[B - 1:B, NH - 1:NH]
+    assert_matches_oracle(dtype, *(sl(x) for x in (q, k, v, f, i, dh)), h=sl(h), m=sl(m), b=sl(b), grads=[sl(g_) for g_ in grads],
+                          chunk_len=Lc, precise=precise)
