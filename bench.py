@@ -284,7 +284,7 @@ def run_scan(ffi, steps, warmup, backward=False, shape=(1, 4, 2048, 1024), tag="
         step()
     torch.cuda.synchronize()
     ffi.timing_enable(False)
-    names = ("gates", "scan_carry", "scan_state", "scan_out") + (("scan_glue", "gate_bwd", "df") if backward else ())
+    names = ("gates", "scan_carry", "scan_state", "scan_out") + (("scan_glue", "df") if backward else ())
     kern = {name: ffi.timing_read(name) for name in names}
     ms_step = (t1 - t0) * 1e3 / steps
     BH = B * NH

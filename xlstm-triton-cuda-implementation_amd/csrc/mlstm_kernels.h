@@ -261,10 +261,29 @@ struct ScanArgs {
     int BH, S, D, NC;
     // What the last kernel writes to h: 0 = silu(o) * numerator / n (the scan form's output), 1 = numerator / n (ungated),
     // 2 = the numerator itself, sum_j exp(a_j - A_t) (q_t . k_j) / sqrt(D) v_j: the causal weighted sum the backward pass
-    // reuses with other operands in the places of q, k and v.  Bout (may be null): the normaliser sums b_t, modes 0 and 1.
+    // reuses with other operands in the places of q, k and v, finished as `ep` says.  Bout (may be null): the normaliser
+    // sums b_t, modes 0 and 1.
     int finish_mode;
     float* Bout;
     float* Hun;           // mode 0 only, may be null: numerator / n next to the gated output (what a backward wants kept)
+    // rev (mode 2 only): q, k and v hold the sequence in its own order and the pipeline walks it from the end: position t
+    // of the walk is row S-1-t of q, k and v.  Gate arrays, P, Nst, h and hpart are in walk order.
+    int rev;
+    // Mode 2 can carry a vector sum along with the matrix one (ep.vec):
+    //   numerator_t = sum_{j<=t} exp(a_j - A_t) / sqrt(D) ((q_t . k_j) + rs_t cs_j) v_j
+    // rs = ep.row_scale ([BH,S], walk order; null: 1), cs = col_scale ([BH,S], in the order of the rows of q, k, v; null: 1).
+    // The pairs inside a chunk take the term into their weights P; the chunks before it come through Nst, which then holds
+    // sum_j exp(a_j - A_end) / sqrt(D) cs_j v_j at the chunk ends.  What the last kernel then does with row t:
+    //   x = numerator_t (+ rs_t decay_t Nst_{c-1}),  x *= exp2(wd_alpha2_j - wd_beta2_j)  (gate arrays of the output row j; may be null)
+    //   out_j = x  with j = t, or S-1-t when out_rev             (out null: h, in place; out_rev needs out != h)
+    //   dot_out_j = dot_with_j . x,  x_out_j = dot_out_j - dot_minus_j                              (each may be null)
+    const float* col_scale;
+    struct Epilogue {
+        float* out; int out_rev;
+        int vec; const float* row_scale;
+        const float* wd_alpha2; const float* wd_beta2;
+        const float* dot_with; float* dot_out; const float* dot_minus; float* x_out;
+    } ep;
     // segments of the sequence that the state kernel runs side by side (filled in by launch_scan from scan_segments);
     // seg_state: scan_segment_state_bytes() bytes of scratch for the states at the segment ends, needed when nseg > 1
     float* seg_state;

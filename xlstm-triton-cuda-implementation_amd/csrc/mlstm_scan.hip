@@ -27,31 +27,53 @@ __device__ __forceinline__ f32x16 mma_f32(float a, float b, f32x16 c) { return _
 
 // ---------------------------------------------------------------------------------------------------------------
 // Four workgroups per (head, chunk): three form one 32x32 block of P each (the head dimension split over the four
-// waves, summed through LDS), the fourth clears the masked block and forms the chunk's contribution to n~.
+// waves, summed through LDS), the fourth clears the masked block and forms the chunk's contribution to n~ (mode 2: to the
+// vector sum that rides along, over the rows of v, if there is one).
 template <int D>
 __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
     __shared__ float red[4][16][64];
-    const int role = blockIdx.x & 3, c = (blockIdx.x >> 2) % a.NC, bh = (blockIdx.x >> 2) / a.NC;
+    // Consecutive workgroups go to the eight XCDs in turn; the four roles of a chunk read the same rows of q and k, so
+    // they take workgroups of one XCD (eight apart), which share an L2.
+    int role, cidx;
+    if ((gridDim.x & 31) == 0) {
+        const int xcd = blockIdx.x & 7, r = blockIdx.x >> 3;
+        role = r & 3; cidx = (r >> 2) * 8 + xcd;
+    } else {
+        role = blockIdx.x & 3; cidx = blockIdx.x >> 2;
+    }
+    const int c = cidx % a.NC, bh = cidx / a.NC;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
     const int S = a.S;
     const size_t hoff = (size_t)bh * S, poff = (size_t)bh * a.NC * GRAN;
     float* P = a.P + ((size_t)bh * a.NC + c) * GRAN * GRAN;
     const float log2scale = -0.5f * __log2f((float)D);
+    auto row_of = [&](int t) { return hoff + (a.rev ? S - 1 - t : t); };   // the row of q, k, v that holds walk position t < S
+    const bool mode2 = a.finish_mode == 2, vec = mode2 && a.ep.vec;
     if (role == 3) {
         float* sw = &red[0][0][0];
-        if (tid < GRAN) sw[tid] = fast_exp2(a.alpha2[poff + GRAN * c + tid] - a.beta2[poff + GRAN * c + GRAN - 1] + log2scale);
         for (int i = tid; i < 32 * 32; i += 256) P[(i >> 5) * GRAN + 32 + (i & 31)] = 0.f;  // queries 0..31, keys 32..63
+        if (mode2 && !vec) return;
+        if (tid < GRAN) {
+            float w = fast_exp2(a.alpha2[poff + GRAN * c + tid] - a.beta2[poff + GRAN * c + GRAN - 1] + log2scale);
+            if (vec && a.col_scale) w *= a.col_scale[row_of(GRAN * c + tid < S ? GRAN * c + tid : S - 1)];
+            sw[tid] = w;
+        }
         __syncthreads();
+        const float* const src = mode2 ? a.v : a.k;
         float* dn = a.Nst + ((size_t)bh * a.NC + c) * D;  // dn[k] = sum_j w_j K[j][k]   (w_j = 0 for padded positions)
-        for (int k = tid; k < D; k += 256) {
-            float s0 = 0.f, s1 = 0.f;
-#pragma unroll 8
-            for (int j = 0; j < GRAN; j += 2) {
-                int j0 = GRAN * c + j, j1 = j0 + 1;
+        for (int k = tid; k < D; k += 256) {   // (the column's 64 loads are issued together: the loop is bound by their latency)
+            float kv[GRAN];
+#pragma unroll
+            for (int j = 0; j < GRAN; j++) {
+                int j0 = GRAN * c + j;
                 j0 = j0 < S ? j0 : S - 1;
-                j1 = j1 < S ? j1 : S - 1;
-                s0 += sw[j] * a.k[(hoff + j0) * D + k];
-                s1 += sw[j + 1] * a.k[(hoff + j1) * D + k];
+                kv[j] = src[row_of(j0) * D + k];
+            }
+            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+            for (int j = 0; j < GRAN; j += 2) {
+                s0 += sw[j] * kv[j];
+                s1 += sw[j + 1] * kv[j + 1];
             }
             dn[k] = s0 + s1;
         }
@@ -65,8 +87,8 @@ __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
         int t = GRAN * c + 32 * tb + c32, j = GRAN * c + 32 * jb + c32;
         t = t < S ? t : S - 1;
         j = j < S ? j : S - 1;
-        const float* qrow = a.q + (hoff + t) * D + wave * (D / 4) + 4 * h;
-        const float* krow = a.k + (hoff + j) * D + wave * (D / 4) + 4 * h;
+        const float* qrow = a.q + row_of(t) * D + wave * (D / 4) + 4 * h;
+        const float* krow = a.k + row_of(j) * D + wave * (D / 4) + 4 * h;
 #pragma unroll 8
         for (int s = 0; s < D / 32; s++) {
             const f32x4 qv = *reinterpret_cast<const f32x4*>(qrow + 8 * s);
@@ -81,29 +103,45 @@ __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
     // accumulator: column (key) = 32*jb + c32, rows (queries) 32*tb + 8*(r/4) + 4h + r%4; wave w finishes r = 4w..4w+3
     const int jl = 32 * jb + c32;
     const float alj = a.alpha2[poff + GRAN * c + jl];
+    const float cs = !vec ? 0.f : (a.col_scale ? a.col_scale[row_of(GRAN * c + jl < S ? GRAN * c + jl : S - 1)] : 1.0f);
 #pragma unroll
     for (int e = 0; e < 4; e++) {
         const int r = 4 * wave + e;
         const int tl = 32 * tb + 8 * (r >> 2) + 4 * h + (r & 3);
-        const float sum = red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane];
+        float sum = red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane];
+        if (vec) sum += cs * (a.ep.row_scale ? a.ep.row_scale[hoff + (GRAN * c + tl < S ? GRAN * c + tl : S - 1)] : 1.0f);
         float p = sum * fast_exp2(alj - a.beta2[poff + GRAN * c + tl] + log2scale);
         if (jl > tl) p = 0.f;
         P[tl * GRAN + jl] = p;
     }
 }
 
-// n~_c = gamma_c n~_{c-1} + dn_c over the chunks of a head, in place
+// n~_c = gamma_c n~_{c-1} + dn_c over the chunks of a head, in place.  One thread per column; the decays of 256 chunks at
+// a time are formed side by side, and the column's sums are fetched eight chunks ahead of the serial sum.
 __global__ __launch_bounds__(256) void scan_ncarry_kernel(ScanArgs a) {
-    const int bh = blockIdx.y, k = blockIdx.x * 256 + threadIdx.x;
-    if (k >= a.D) return;
-    const size_t poff = (size_t)bh * a.NC * GRAN;
-    float* n = a.Nst + (size_t)bh * a.NC * a.D + k;
-    float run = n[0];
-    for (int c = 1; c < a.NC; c++) {
-        const float gam = fast_exp2(a.beta2[poff + GRAN * c - 1] - a.beta2[poff + GRAN * c + GRAN - 1] +
-                                    (float)(a.G2[(size_t)bh * a.NC + c] - a.G2[(size_t)bh * a.NC + c - 1]));
-        run = gam * run + n[(size_t)c * a.D];
-        n[(size_t)c * a.D] = run;
+    __shared__ float sgam[256];
+    const int bh = blockIdx.y, tid = threadIdx.x, k = blockIdx.x * 256 + tid, NC = a.NC;
+    const bool mine = k < a.D;
+    const size_t poff = (size_t)bh * NC * GRAN;
+    float* n = a.Nst + (size_t)bh * NC * a.D + (mine ? k : 0);
+    float run = mine ? n[0] : 0.f;
+    for (int c0 = 1; c0 < NC; c0 += 256) {
+        __syncthreads();
+        if (const int c = c0 + tid; c < NC)
+            sgam[tid] = fast_exp2(a.beta2[poff + GRAN * c - 1] - a.beta2[poff + GRAN * c + GRAN - 1] +
+                                  (float)(a.G2[(size_t)bh * NC + c] - a.G2[(size_t)bh * NC + c - 1]));
+        __syncthreads();
+        const int cn = NC - c0 < 256 ? NC - c0 : 256;
+        for (int cb = 0; cb < cn && mine; cb += 8) {
+            float x[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) x[j] = cb + j < cn ? n[(size_t)(c0 + cb + j) * a.D] : 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                run = (cb + j < cn ? sgam[cb + j] : 1.0f) * run + x[j];
+                if (cb + j < cn) n[(size_t)(c0 + cb + j) * a.D] = run;
+            }
+        }
     }
 }
 
@@ -123,7 +161,9 @@ template <> struct FVec<1> { struct type { float x; __device__ float operator[](
 //                       state at its end (accumulator registers as they are) in seg_state;
 //   scan_segcarry_kernel turns those into the true states at the segment ends (a short serial sum over the segments);
 //   STATE_ONLY = false  the walk proper: segment s > 0 starts from the state at the end of segment s - 1.
-template <int D, int KS, int NW, bool STATE_ONLY>
+// REV: q, k and v are walked from their last row (ScanArgs::rev).  A complete chunk's 64 rows then lie in front of the row of
+// its first position; the lane parts of the addresses stay non-negative by counting from the chunk's last position.
+template <int D, int KS, int NW, bool STATE_ONLY, bool REV>
 __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     constexpr int KPW = D / KS / NW, NKB = KPW / 32, NVT = D / 32;  // key columns per wave, in blocks of 32
     constexpr int SH = 32 / (NW * KS);                              // in-chunk contraction steps per wave
@@ -146,8 +186,10 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     float* out = (ks == 0 ? a.h : a.hpart + (size_t)(ks - 1) * a.BH * S * D) + hoff * D;
     const int kbase = (ks * NW + wave) * KPW, v0 = 32 * vt;
     const float log2scale = -0.5f * __log2f((float)D);
-    const int v_lofs = 32 * h * D + v0 + c32;             // lane part of a value address (row 32h, column v0 + c32)
-    const int k_lofs = 32 * h * D + kbase + NKB * c32;    // lane part of a key address
+    const int hrow = REV ? 32 * (1 - h) : 32 * h;         // the lane half's first row in a chunk's 64 rows as they lie in memory
+    const int v_lofs = hrow * D + v0 + c32;               // lane part of a value address (column v0 + c32)
+    const int k_lofs = hrow * D + kbase + NKB * c32;      // lane part of a key address
+    auto row_of = [&](int t) { return (size_t)(REV ? S - 1 - t : t); };   // the row that holds walk position t < S
 
     // Gate vectors of a chunk: weights of its keys, decays of its queries (from the previous chunk end).  The carried
     // state is kept as st = C~ / Gamma with a running power of two Gamma <= 1, so that the per-chunk decay gamma_c
@@ -195,7 +237,7 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
     auto load_q = [&](int c, int tb, int x, int e) {  // (row clamped: the chunk may be the partial one)
         int t = GRAN * c + 32 * tb + c32;
         t = t < S ? t : S - 1;
-        qreg[tb][x][e] = *reinterpret_cast<const kvec*>(Q + (size_t)t * D + kbase + 4 * NKB * h + NKB * (8 * x + e));
+        qreg[tb][x][e] = *reinterpret_cast<const kvec*>(Q + row_of(t) * D + kbase + 4 * NKB * h + NKB * (8 * x + e));
     };
     if constexpr (!STATE_ONLY) {
 #pragma unroll
@@ -223,18 +265,20 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
         float pa[2][SH];
         float vin[SH];  // this wave's values for the in-chunk products (a register array takes no wave-dependent index)
         kvec kreg[32];
-        const float* vrow = V + (size_t)t0 * D;  // uniform
-        const float* krow = K + (size_t)t0 * D;  // uniform
-        auto load_v = [&](int s) {
+        // uniform: the first of the chunk's 64 rows in memory (REV: the row of its last position; only complete chunks use it)
+        const size_t r0 = LAST ? 0 : (REV ? (size_t)(S - GRAN - t0) : (size_t)t0);
+        const float* vrow = V + r0 * D;
+        const float* krow = K + r0 * D;
+        auto load_v = [&](int s) {   // position t0 + 32h + s
             if constexpr (LAST) {
                 int j = t0 + 32 * h + s;
                 j = j < S ? j : S - 1;
-                vraw[s] = V[(size_t)j * D + v0 + c32];
+                vraw[s] = V[row_of(j) * D + v0 + c32];
             } else {
-                vraw[s] = (vrow + (size_t)s * D)[v_lofs];
+                vraw[s] = (vrow + (size_t)(REV ? 31 - s : s) * D)[v_lofs];
             }
         };
-        auto load_k = [&](int s) { kreg[s] = *reinterpret_cast<const kvec*>(krow + (size_t)s * D + k_lofs); };
+        auto load_k = [&](int s) { kreg[s] = *reinterpret_cast<const kvec*>(krow + (size_t)(REV ? 31 - s : s) * D + k_lofs); };
         // ---- read-out of the carried state: acc[tb] = decay_t * Q_c[32 tb.., k-range of this wave] . C~^T
         f32x16 acc[2];
 #pragma unroll
@@ -263,7 +307,7 @@ __global__ __launch_bounds__(NW * 64) void scan_state_kernel(ScanArgs a) {
             for (int s = 0; s < SH; s++) {
                 int j = t0 + 32 * h + s0 + s;
                 if constexpr (LAST) j = j < S ? j : S - 1;
-                vin[s] = V[(size_t)j * D + v0 + c32];
+                vin[s] = V[row_of(j) * D + v0 + c32];
             }
         };
 #pragma unroll
@@ -392,6 +436,43 @@ __global__ __launch_bounds__(256) void scan_finish_kernel(ScanArgs a, int KS) {
     for (size_t row = (size_t)blockIdx.x * 4 + wave; row < rows; row += (size_t)gridDim.x * 4) {
         const int bh = (int)(row / a.S), t = (int)(row % a.S), c = t / GRAN;
         const size_t poff = (size_t)bh * a.NC * GRAN;
+        if (a.finish_mode == 2) {
+            const ScanArgs::Epilogue& ep = a.ep;
+            const size_t orow = ep.out_rev ? (size_t)bh * a.S + (a.S - 1 - t) : row;
+            const bool carried = ep.vec && c > 0;
+            // rs_t decay_t, the factor of the vector sum at the end of the chunk before
+            const float cf = !carried ? 0.f : (ep.row_scale ? ep.row_scale[row] : 1.0f) *
+                                                  fast_exp2(a.beta2[poff + GRAN * c - 1] - a.beta2[poff + t] +
+                                                            (float)(a.G2[(size_t)bh * a.NC + c] - a.G2[(size_t)bh * a.NC + c - 1]));
+            const float* cr = carried ? a.Nst + ((size_t)bh * a.NC + c - 1) * D : nullptr;
+            const float wd = ep.wd_alpha2 ? fast_exp2(ep.wd_alpha2[poff + (orow - (size_t)bh * a.S)] - ep.wd_beta2[poff + (orow - (size_t)bh * a.S)]) : 1.0f;
+            float* const dst = (ep.out ? ep.out : a.h) + orow * D;
+            float acc = 0.f;
+            for (int k = 4 * lane; k < D; k += 256) {
+                f32x4 x = *reinterpret_cast<const f32x4*>(a.h + row * D + k);
+                for (int p = 1; p < KS; p++) x += *reinterpret_cast<const f32x4*>(a.hpart + ((size_t)(p - 1) * rows + row) * D + k);
+                if (carried) {
+                    const f32x4 cv = *reinterpret_cast<const f32x4*>(cr + k);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[e] += cf * cv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) x[e] *= wd;
+                if (ep.dot_with) {
+                    const f32x4 dv = *reinterpret_cast<const f32x4*>(ep.dot_with + orow * D + k);
+                    acc += dv[0] * x[0] + dv[1] * x[1] + dv[2] * x[2] + dv[3] * x[3];
+                }
+                *reinterpret_cast<f32x4*>(dst + k) = x;
+            }
+            if (ep.dot_with) {
+                acc = wave_reduce<OpAdd>(acc);
+                if (lane == 0) {
+                    ep.dot_out[orow] = acc;
+                    if (ep.x_out) ep.x_out[orow] = acc - ep.dot_minus[orow];
+                }
+            }
+            continue;
+        }
         float dot = 0.f;
         if (c > 0) {
             const float* n = a.Nst + ((size_t)bh * a.NC + c - 1) * D;
@@ -407,7 +488,7 @@ __global__ __launch_bounds__(256) void scan_finish_kernel(ScanArgs a, int KS) {
         }
         const float prow = a.P[((size_t)bh * a.NC + c) * GRAN * GRAN + (size_t)(t - GRAN * c) * GRAN + lane];
         const float b = dot + wave_reduce<OpAdd>(prow);
-        const float inv = a.finish_mode == 2 ? 1.0f : 1.0f / (fmaxf(fabsf(b), __expf(-a.M[row])) + 1e-6f);
+        const float inv = 1.0f / (fmaxf(fabsf(b), __expf(-a.M[row])) + 1e-6f);
         if (a.Bout && lane == 0) a.Bout[row] = b;
         for (int k = 4 * lane; k < D; k += 256) {
             f32x4 x = *reinterpret_cast<const f32x4*>(a.h + row * D + k);
@@ -431,35 +512,36 @@ __global__ __launch_bounds__(256) void scan_finish_kernel(ScanArgs a, int KS) {
     }
 }
 
-template <int D, int KS, int NW>
+template <int D, int KS, int NW, bool REV>
 static void launch_state(const ScanArgs& a, hipStream_t st) {
     if constexpr ((D / KS / NW == 32 || D / KS / NW == 64 || D / KS / NW == 128) && NW * KS <= 32) {
         constexpr int lds_bytes = (2 * NW * 32 * 64 + 3 * 2 * GRAN) * 4;
         // (a failure here shows up as a launch error, which the caller reads with hipGetLastError)
-        (void)lds_limit_once<scan_state_kernel<D, KS, NW, false>>(lds_bytes);
+        (void)lds_limit_once<scan_state_kernel<D, KS, NW, false, REV>>(lds_bytes);
         const int wgs = a.BH * (D / 32) * KS;
         if (a.nseg > 1) {
-            (void)lds_limit_once<scan_state_kernel<D, KS, NW, true>>(lds_bytes);
-            hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, true>), dim3(wgs, a.nseg - 1), dim3(NW * 64), lds_bytes, st, a);
+            (void)lds_limit_once<scan_state_kernel<D, KS, NW, true, REV>>(lds_bytes);
+            hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, true, REV>), dim3(wgs, a.nseg - 1), dim3(NW * 64), lds_bytes, st, a);
             const size_t elems = (size_t)wgs * NW * (D / KS / NW / 32) * 16 * 64;   // = BH * D * D
             hipLaunchKernelGGL(scan_segcarry_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, st, a, elems,
                                NW * (D / KS / NW / 32) * 16 * 64);
         }
-        hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, false>), dim3(wgs, a.nseg), dim3(NW * 64), lds_bytes, st, a);
+        hipLaunchKernelGGL((scan_state_kernel<D, KS, NW, false, REV>), dim3(wgs, a.nseg), dim3(NW * 64), lds_bytes, st, a);
     }
 }
 
 template <int D, int KS>
 static void launch_state_w(const ScanArgs& a, int NW, hipStream_t st) {
     (void)NW;  // scan_plan: two waves per workgroup at D = 64, four above
-    launch_state<D, KS, (D / 32 < 4 ? D / 32 : 4)>(a, st);
+    if (a.rev) launch_state<D, KS, (D / 32 < 4 ? D / 32 : 4), true>(a, st);
+    else launch_state<D, KS, (D / 32 < 4 ? D / 32 : 4), false>(a, st);
 }
 
 template <int D>
 static int launch_scan_d(const ScanArgs& a, int KS, int NW, hipStream_t st, void (*mark)(int, hipStream_t, bool)) {
     mark(MLSTM_K_SCAN_CARRY, st, true);
     hipLaunchKernelGGL(scan_intra_kernel<D>, dim3(a.BH * a.NC * 4), dim3(256), 0, st, a);
-    hipLaunchKernelGGL(scan_ncarry_kernel, dim3((D + 255) / 256, a.BH), dim3(256), 0, st, a);
+    if (a.finish_mode != 2 || a.ep.vec) hipLaunchKernelGGL(scan_ncarry_kernel, dim3((D + 255) / 256, a.BH), dim3(256), 0, st, a);
     mark(MLSTM_K_SCAN_CARRY, st, false);
     mark(MLSTM_K_SCAN_STATE, st, true);
     if (KS == 8) launch_state_w<D, 8>(a, NW, st);
@@ -511,6 +593,11 @@ int launch_scan(const ScanArgs& a_in, int KS, hipStream_t st, void (*mark)(int, 
     ScanArgs a = a_in;
     scan_segments(a.BH, a.S, a.D, &a.nseg, &a.seg_chunks);
     if (a.nseg > 1 && !a.seg_state) return MLSTM_EWORKSPACE;
+    if (a.finish_mode != 2 && (a.rev || a.col_scale)) return MLSTM_EINVAL;
+    if (a.finish_mode == 2 && ((a.ep.out_rev && (!a.ep.out || a.ep.out == a.h)) ||
+                               (a.ep.dot_with && !a.ep.dot_out) || (a.ep.x_out && !(a.ep.dot_with && a.ep.dot_minus)) ||
+                               (!a.ep.wd_alpha2 != !a.ep.wd_beta2)))
+        return MLSTM_EINVAL;
     int ks, NW; scan_plan(a.BH, a.D, &ks, &NW);
     if (NW != (a.D / 32 < 4 ? a.D / 32 : 4)) return MLSTM_ESHAPE;
     const int kpw = a.D / KS / NW;
