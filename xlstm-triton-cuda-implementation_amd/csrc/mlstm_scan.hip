@@ -29,9 +29,18 @@ __device__ __forceinline__ f32x16 mma_f32(float a, float b, f32x16 c) { return _
 // Four workgroups per (head, chunk): three form one 32x32 block of P each (the head dimension split over the four
 // waves, summed through LDS), the fourth clears the masked block and forms the chunk's contribution to n~ (mode 2: to the
 // vector sum that rides along, over the rows of v, if there is one).
+// The products' operands want one row per lane, which from memory would be 32 bytes per row and instruction; so a wave
+// fetches its quarter of the head dimension in blocks of FBW columns with whole 128-byte lines per row (four blocks in
+// flight), passes them through a piece of LDS of its own (rows padded by four floats: conflict-free both ways) and reads
+// the operands from there.
 template <int D>
 __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
-    __shared__ float red[4][16][64];
+    constexpr int DW = D / 4, FBW = DW < 32 ? DW : 32, NB = DW / FBW;   // columns per wave, per block; blocks
+    constexpr int LPR = FBW / 4, RPI = 64 / LPR, NLD = LPR;             // lanes per row, rows per load instruction, loads per block
+    constexpr int LST = FBW + 4, PD = NB < 4 ? NB : 4;                  // LDS row stride (floats); blocks in flight
+    __shared__ __align__(16) float stage[4][64 * LST];                  // per wave: 32 rows of q, then 32 rows of k
+    static_assert(64 * LST >= 16 * 64, "the partial sums reuse a wave's stage");
+    auto red_at = [&](int w, int r, int l) -> float& { return stage[w][r * 64 + l]; };
     // Consecutive workgroups go to the eight XCDs in turn; the four roles of a chunk read the same rows of q and k, so
     // they take workgroups of one XCD (eight apart), which share an L2.
     int role, cidx;
@@ -50,7 +59,7 @@ __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
     auto row_of = [&](int t) { return hoff + (a.rev ? S - 1 - t : t); };   // the row of q, k, v that holds walk position t < S
     const bool mode2 = a.finish_mode == 2, vec = mode2 && a.ep.vec;
     if (role == 3) {
-        float* sw = &red[0][0][0];
+        float* sw = &stage[0][0];
         for (int i = tid; i < 32 * 32; i += 256) P[(i >> 5) * GRAN + 32 + (i & 31)] = 0.f;  // queries 0..31, keys 32..63
         if (mode2 && !vec) return;
         if (tid < GRAN) {
@@ -84,21 +93,45 @@ __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.f;
     {
-        int t = GRAN * c + 32 * tb + c32, j = GRAN * c + 32 * jb + c32;
-        t = t < S ? t : S - 1;
-        j = j < S ? j : S - 1;
-        const float* qrow = a.q + row_of(t) * D + wave * (D / 4) + 4 * h;
-        const float* krow = a.k + row_of(j) * D + wave * (D / 4) + 4 * h;
-#pragma unroll 8
-        for (int s = 0; s < D / 32; s++) {
-            const f32x4 qv = *reinterpret_cast<const f32x4*>(qrow + 8 * s);
-            const f32x4 kv = *reinterpret_cast<const f32x4*>(krow + 8 * s);
+        float* const stg = stage[wave];
+        const int lrow = lane / LPR, lcol = 4 * (lane % LPR);
+        const float* src[NLD];   // this lane's rows: load i covers stage rows RPI*i .. RPI*i + RPI-1 (0..31: q, 32..63: k)
 #pragma unroll
-            for (int e = 0; e < 4; e++) acc = mma_f32(qv[e], kv[e], acc);  // rows = queries, columns = keys
+        for (int i = 0; i < NLD; i++) {
+            const int r = RPI * i + lrow;
+            int t = GRAN * c + (r < 32 ? 32 * tb + r : 32 * jb + r - 32);
+            t = t < S ? t : S - 1;
+            src[i] = (r < 32 ? a.q : a.k) + row_of(t) * D + wave * DW + lcol;
+        }
+        f32x4 rg[PD][NLD];
+#pragma unroll
+        for (int b = 0; b < PD; b++)
+#pragma unroll
+            for (int i = 0; i < NLD; i++) rg[b][i] = *reinterpret_cast<const f32x4*>(src[i] + b * FBW);
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) *reinterpret_cast<f32x4*>(stg + (RPI * i + lrow) * LST + lcol) = rg[b % PD][i];
+            if (b + PD < NB) {
+#pragma unroll
+                for (int i = 0; i < NLD; i++) rg[b % PD][i] = *reinterpret_cast<const f32x4*>(src[i] + (b + PD) * FBW);
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int s = 0; s < FBW / 8; s++) {
+                const f32x4 qv = *reinterpret_cast<const f32x4*>(stg + c32 * LST + 8 * s + 4 * h);
+                const f32x4 kv = *reinterpret_cast<const f32x4*>(stg + (32 + c32) * LST + 8 * s + 4 * h);
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc = mma_f32(qv[e], kv[e], acc);  // rows = queries, columns = keys
+            }
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
         }
     }
+    __syncthreads();   // (every wave is done with its stage: the partial sums go there)
 #pragma unroll
-    for (int r = 0; r < 16; r++) red[wave][r][lane] = acc[r];
+    for (int r = 0; r < 16; r++) red_at(wave, r, lane) = acc[r];
     __syncthreads();
     // accumulator: column (key) = 32*jb + c32, rows (queries) 32*tb + 8*(r/4) + 4h + r%4; wave w finishes r = 4w..4w+3
     const int jl = 32 * jb + c32;
@@ -108,7 +141,7 @@ __global__ __launch_bounds__(256) void scan_intra_kernel(ScanArgs a) {
     for (int e = 0; e < 4; e++) {
         const int r = 4 * wave + e;
         const int tl = 32 * tb + 8 * (r >> 2) + 4 * h + (r & 3);
-        float sum = red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane];
+        float sum = red_at(0, r, lane) + red_at(1, r, lane) + red_at(2, r, lane) + red_at(3, r, lane);
         if (vec) sum += cs * (a.ep.row_scale ? a.ep.row_scale[hoff + (GRAN * c + tl < S ? GRAN * c + tl : S - 1)] : 1.0f);
         float p = sum * fast_exp2(alj - a.beta2[poff + GRAN * c + tl] + log2scale);
         if (jl > tl) p = 0.f;
