@@ -253,7 +253,7 @@ int mlstm_scan_backward_ex(const void* dh_gated, const void* q, const void* k, c
                            int D, int dtype, void* workspace, size_t workspace_bytes, void* stream);
 /* The same pair for a training step that keeps what its backward would otherwise form again: the forward also leaves the
  * ungated output h_ungated ([B,NH,S,D] fp32: numerator / n, before silu(o)) and the normaliser sums b ([B,NH,S]); the backward
- * that is handed both skips its forward pass (one of its five walks over the sequence) and returns the same bits.  Null
+ * that is handed both skips its forward pass (one of its four walks over the sequence) and returns the same bits.  Null
  * h_ungated and b make mlstm_scan_backward_saved_ex identical to mlstm_scan_backward_ex. */
 int mlstm_scan_forward_save_ex(const void* q, const void* k, const void* v, const void* f, const void* i, const void* o, void* h,
                                void* h_ungated, float* b, int B, int NH, int S, int D, int dtype, void* workspace,
