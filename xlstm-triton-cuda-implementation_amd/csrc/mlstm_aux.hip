@@ -130,7 +130,11 @@ __global__ __launch_bounds__(1024) void dfchunk_kernel(const TG* __restrict__ F,
         const int g = t / GRAN, g0 = c * (chunk_len / GRAN);
         const float* rp = rowpart + (size_t)bh * RS * S + t;     // slice = key tile - first tile of the chunk
         float row = rowinter[(size_t)bh * S + t];
-        for (int j = g0; j <= g; j++) row += rp[(size_t)(j - g0) * S];
+        float part[16];   // (a fixed count, so that the loads leave together: chunk_len <= 1024 is at most 16 slices)
+#pragma unroll
+        for (int j = 0; j < 16; j++) part[j] = j <= g - g0 ? rp[(size_t)j * S] : 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; j++) row += part[j];
         col = colsum[(size_t)bh * S + t];
         f = (float)F[lg.head(bh) + (size_t)t * lg.ss];
         v = col - row;

@@ -81,7 +81,7 @@ __device__ __forceinline__ float forget_log(const TG* f, size_t ss, int t, int f
     return t > 0 ? x - (float)f[(size_t)(t - 1) * ss] : x;
 }
 
-// Sequences of up to 16 * GPW granules: every wave keeps its granules' cumulative sums and alphas in registers
+// Sequences of up to 16 * GPW granules (GPW = 4, 8, 16: S <= 16384): every wave keeps its granules' cumulative sums and alphas in registers
 // between the two passes, and issues all its loads before the first scan (one memory round trip instead of one per granule
 // and pass).
 template <typename TG, int GPW>
@@ -174,6 +174,8 @@ static hipError_t launch_gates_t(const void* F, const void* I, float* alpha2, fl
         hipLaunchKernelGGL((gates_kernel_reg<TG, 4>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     else if (NG <= 16 * 8)
         hipLaunchKernelGGL((gates_kernel_reg<TG, 8>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
+    else if (NG <= 16 * 16)
+        hipLaunchKernelGGL((gates_kernel_reg<TG, 16>), dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     else
         hipLaunchKernelGGL(gates_kernel<TG>, dim3(BH), dim3(1024), 0, st, (const TG*)F, (const TG*)I, alpha2, beta2, G2, M, ek2, amax2, S, NG, lg, form, stamp);
     return hipGetLastError();
