@@ -17,6 +17,9 @@
 //   scan_finish_kernel  per row: b_t = decay_t (n~_{c-1} . q_t) + rowsum_t(P_c),
 //                       h = (sum of partial numerators) / (max(|b|, exp(-m)) + 1e-6) * silu(o)   (mlstm_scan.py:273-277).
 // HBM traffic: the compulsory stream of q, k, v, o, h, one round trip of the numerator per key range, q once more.
+// The same four kernels evaluate the causal weighted sums of the backward (mlstm_scan_bwd.hip) with other operands in the
+// places of q, k and v: ScanArgs::finish_mode 2 leaves the numerator itself, ScanArgs::rev walks the operands from their
+// last row, ScanArgs::Epilogue says what rides along (a vector sum) and what the last kernel does with a row.
 #include "mlstm_device.h"
 #include "mlstm_kernels.h"
 #include <type_traits>
