@@ -165,6 +165,23 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
                                        P(df), P(di), B, NH, S, D, dt_code, gate_code, P(ws), ws_n, st)
         ffi.check_rc(rc, "mlstm_backward_saved_ex")
 
+    # The per-kernel breakdown comes first: steps of its own with every kernel bracketed by HIP events, outside the timed
+    # region (a few unbracketed ones ahead of them, so that the first launches' one-time costs stay out of the averages).
+    # At least 50, for steady averages; behind them the GPU's clock has settled as well, which a short run straight from
+    # idle does not reach (the first tens of steps after idle run 5-10 % slower) -- `breakdown_steps` in the output says
+    # how many ran.
+    breakdown_steps = max(steps // 4, 50)
+    for _ in range(3):
+        step()
+    torch.cuda.synchronize()
+    ffi.timing_select(None, every=1)
+    ffi.timing_enable(True)
+    for _ in range(breakdown_steps):
+        step()
+    torch.cuda.synchronize()
+    ffi.timing_enable(False)
+    kern = {kname: ffi.timing_read(kname) for kname in ("gates", "chunk_states", "row_fwd", "row_dq", "df")}
+    ffi.timing_read("col")
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -177,16 +194,9 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
         step()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    kern = {"col": ffi.timing_read("col")}
-    # the other kernels' durations, for the breakdown: a few more steps, outside the timed region, all kernels timed
-    ffi.timing_select(None, every=1)
-    for _ in range(max(steps // 4, 1)):
-        step()
-    torch.cuda.synchronize()
     ffi.timing_enable(False)
-    for kname in ("gates", "chunk_states", "row_fwd", "row_dq", "df"):
-        kern[kname] = ffi.timing_read(kname)
-    ffi.timing_read("col")
+    kern["col"] = ffi.timing_read("col")
+    ffi.timing_select(None, every=1)
     kern = {kname: kern[kname] for kname in ("gates", "chunk_states", "row_fwd", "col", "row_dq", "df")}
     assert L.mlstm_kernel_error() == 0, "a kernel's bounded wait expired during the benchmark"
 
@@ -215,7 +225,7 @@ def run_matmul(ffi, name, steps, warmup, precise=False, host=None):
     out = {
         "metric": "mLSTM matmul-form fwd+bwd, time to solution as parallel-form TFLOP/s (7*D*S*(S+1) flops per head; not a hardware "
                   "rate: see executed_tflops) and tokens/s, " + name + (" split mode" if precise else ""),
-        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup, "breakdown_steps": breakdown_steps,
         "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": DTYPE_NAME[dtype], "data": "synthetic",
         "config": {"workload": name, "B": B, "NH": NH, "S": S, "D": D, "f": f"N({f_mean},1)", "i": f"N({i_mean},1)",
