@@ -59,6 +59,11 @@ def test_workspace_sizes_and_argument_errors_need_no_gpu():
     assert 0 < fwd < bwd and scan > 0
     assert L.mlstm_workspace_bytes(ffi.OP_FORWARD_GATED, 4, 8, 4096, 256, ffi.BF16) == fwd
     assert L.mlstm_workspace_bytes(ffi.OP_BACKWARD_GATED, 4, 8, 4096, 256, ffi.BF16) > bwd + 2 * 4 * 8 * 4096 * 256 * 2
+    # the scan form's backward walks q, k, v in place from the end and keeps two [BH,S,D] buffers of its own (plus the partial
+    # numerators of a second key range at D = 1024): three tensors' worth at the reference's scan shape, not eight
+    tensor = 1 * 4 * 2048 * 1024 * 4
+    scan_bwd = L.mlstm_workspace_bytes(ffi.OP_SCAN_BACKWARD, 1, 4, 2048, 1024, ffi.F32)
+    assert 3 * tensor < scan_bwd < 3 * tensor + 8 * 2**20
     assert L.mlstm_workspace_bytes(ffi.OP_FORWARD, 0, 8, 4096, 256, ffi.BF16) == 0
     assert L.mlstm_workspace_bytes(7, 1, 1, 64, 64, ffi.F32) == 0
     null = ctypes.c_void_p(0)
