@@ -155,6 +155,6 @@ def test_matmul_form_fp32_large_head_dimension_limits():
 
 @pytest.mark.parametrize("S,D", [(4096, 128), (2500, 64)])
 def test_scan_backward_one_long_sequence(S, D):
-    # one head: all five passes of the state kernel run in segments
+    # one head: every pass of the state kernel runs in segments (two of them from the end of the sequence backwards)
     q, k, v, f, i, dh, o = O.make_inputs(1, 1, S, D, torch.float32, seed=S + D, with_o=True)
     check(run_backward(dh, q, k, v, f, i, o), dh, q, k, v, f, i, o)
