@@ -249,8 +249,37 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             }
             if constexpr (MODE == R8_FWD) { bsum[0] += blk0 * er0; bsum[1] += blk1 * er1; }
         };
-        // mode 0: block above the diagonal (P = 0), 1: below, 2: diagonal block
+        // One 32 x 32 block of a tile that the diagonal crosses.  mode (the same in all lanes) 0: the block lies above the
+        // diagonal (P = 0), 1: below it (the factorised weights of weigh_fact), 2: on it (one exp2 per element, masked).
         auto weigh_masked = [&](f32x16& sacc, const float* sal, float crow, int mode, float& bs, float invn, float dbr) {
+            if (mode == 0) {
+#pragma unroll
+                for (int x = 0; x < 16; x++) sacc[x] = 0.f;
+                return;
+            }
+            if (mode == 1) {
+                const float* sek = sal + GRAN;
+                const float er = fast_exp2(crow + sek[GRAN + kh]);
+                const float sc = invn * er, of = dbr * er;
+                float blk = 0.f;
+#pragma unroll
+                for (int a4 = 0; a4 < 4; a4++) {
+                    const f32x4 ek = *reinterpret_cast<const f32x4*>(sek + 32 * kh + 8 * a4 + 4 * h);
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        const int x = 4 * a4 + c;
+                        if constexpr (MODE == R8_FWD) {
+                            const float t = sacc[x] * ek[c];
+                            blk += t;
+                            sacc[x] = t * er;
+                        } else {
+                            sacc[x] = (sacc[x] * sc + of) * ek[c];
+                        }
+                    }
+                }
+                if constexpr (MODE == R8_FWD) bs += blk * er;
+                return;
+            }
 #pragma unroll
             for (int a4 = 0; a4 < 4; a4++) {
                 const f32x4 al = *reinterpret_cast<const f32x4*>(sal + 32 * kh + 8 * a4 + 4 * h);
@@ -258,7 +287,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 for (int c = 0; c < 4; c++) {
                     const int x = 4 * a4 + c;
                     float e = fast_exp2(al[c] + crow);
-                    if (mode == 0 || (mode == 2 && (8 * a4 + 4 * h + c > c32))) e = 0.f;
+                    if (8 * a4 + 4 * h + c > c32) e = 0.f;
                     if constexpr (MODE == R8_FWD) {
                         const float p = sacc[x] * e;
                         bs += p;
