@@ -50,13 +50,17 @@ static void check_tile(const char* what) {
 }
 
 template <int HALF_ROW_BYTES>
-static void check_touch() {
-    constexpr int LINES = row8_touch_lines(HALF_ROW_BYTES);
+static void check_pieces() {
+    // the two lanes of a row load every 16-byte piece of the half row exactly once and stay inside it
+    constexpr int NP = row8_pieces_per_lane(HALF_ROW_BYTES);
+    std::vector<int> seen(HALF_ROW_BYTES / 16, 0);
     for (int h = 0; h < 2; h++)
-        for (int ln = 0; ln < LINES; ln += 2)
-            if (row8_touch_ok(ln, h, LINES))
-                CHECK(row8_touch_offset(ln, h) + 4 <= HALF_ROW_BYTES, "touch of line %d by lane half %d ends at %d of %d bytes", ln, h,
-                      row8_touch_offset(ln, h) + 4, HALF_ROW_BYTES);
+        for (int i = 0; i < NP; i++) {
+            const int o = row8_piece_offset(i, h, HALF_ROW_BYTES);
+            CHECK(o % 16 == 0 && o + 16 <= HALF_ROW_BYTES, "piece %d of lane half %d ends at %d of %d bytes", i, h, o + 16, HALF_ROW_BYTES);
+            seen[o / 16]++;
+        }
+    for (size_t k = 0; k < seen.size(); k++) CHECK(seen[k] == 1, "half row of %d bytes: piece %zu loaded %d times", HALF_ROW_BYTES, k, seen[k]);
 }
 
 int main() {
@@ -71,9 +75,9 @@ int main() {
     check_tile<__bf16, 256, 32, 256>("32-row tile");
     check_tile<__bf16, 128, 128, 256>("128-row tile");
     check_tile<__bf16, 256, 128, 256>("128-row tile");
-    // half rows of the dQ pass's early touch: D = 128 and 256, 16-bit
-    check_touch<128>();
-    check_touch<256>();
+    // half rows of the dQ pass: the pieces its row sums load, D = 128 and 256, 16-bit
+    check_pieces<128>();
+    check_pieces<256>();
     if (failures) { std::printf("tile_bounds: %d check(s) failed\n", failures); return 1; }
     std::printf("tile_bounds: ok\n");
     return 0;

@@ -360,12 +360,11 @@ struct TileDma {
     __device__ __forceinline__ void issue(T* tile, const T* g_tile_v, const Rows& o) const { issue_range(tile, g_tile_v, 0, PER_WAVE, o); }
 };
 
-// Early touch of a row's cache lines by the two lanes (h = 0, 1) that own the row in the eight-wave row kernel: lane h reads
-// one word of line ln + h, ln = 0, 2, ...; a half row of `half_row_bytes` has half_row_bytes / 128 lines and a lane must not
-// go past the last of them (at D = 128 a 16-bit half row is ONE line).  Shared with the host-side bounds check.
-__host__ __device__ constexpr int row8_touch_lines(int half_row_bytes) { return half_row_bytes / 128; }
-__host__ __device__ constexpr bool row8_touch_ok(int ln, int h, int lines) { return ln + h < lines; }
-__host__ __device__ constexpr int row8_touch_offset(int ln, int h) { return 128 * (ln + h); }
+// The 16-byte pieces that the two lanes (h = 0, 1) of a row load of their wave's half row for the row sums q . dQ of the
+// eight-wave row kernel: a half row of `half_row_bytes` has half_row_bytes / 16 pieces, lane h takes the pieces
+// NP h .. NP h + NP - 1 with NP = half of them.  Shared with the host-side bounds check.
+__host__ __device__ constexpr int row8_pieces_per_lane(int half_row_bytes) { return half_row_bytes / 32; }
+__host__ __device__ constexpr int row8_piece_offset(int i, int h, int half_row_bytes) { return 16 * (row8_pieces_per_lane(half_row_bytes) * h + i); }
 
 // 64 floats (one per key of a tile) by the first wave
 __device__ __forceinline__ void vec64_dma(float* dst, const float* src, int tid) {

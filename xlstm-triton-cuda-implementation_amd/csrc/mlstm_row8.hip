@@ -526,22 +526,6 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             if constexpr (MODE == R8_FWD) m_pre[r] = a.M[hoff + rowc[r]];
         }
         y2_bulk(0);
-        // The row sums of the state part need the rows' Q behind the state tiles (q_i . dQ_i): touch the lines now, so that
-        // the loads then find them in the L2 instead of waiting for HBM in the middle of the prologue.  The touched words are
-        // only "used" behind the state tiles: a use here would wait for them, and for every copy issued before them.
-        int touched[2] = {0, 0};
-        if (MODE == R8_DQ && chunk > 0) {
-            const char* qb = reinterpret_cast<const char*>(a.Qrow) + (offA + (size_t)dh * (D / 2)) * sizeof(T);
-            constexpr int LINES = row8_touch_lines((D / 2) * (int)sizeof(T));   // 128-byte lines of this wave's half of a row
-#pragma unroll
-            for (int r = 0; r < 2; r++) {
-#pragma unroll
-                for (int ln = 0; ln < LINES; ln += 2) {
-                    if (row8_touch_ok(ln, h, LINES))   // (the two lanes of a row take a line each; never past the end of the half row)
-                        touched[r] ^= *reinterpret_cast<const int*>(qb + (size_t)rowc[r] * rsA * sizeof(T) + row8_touch_offset(ln, h));
-                }
-            }
-        }
         if (MODE == R8_DQ && chunk == 0) {
             // Per-row scalars of the backward for row block r = dh of the row group (the producers need them from their
             // first tile on, the column kernel reads them from global memory): this role idles until the first P arrives.
@@ -611,22 +595,38 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                     }
             }
             if constexpr (MODE == R8_DQ) {
-                asm volatile("" ::"v"(touched[0]), "v"(touched[1]));
                 // Row sums of dD over the keys before the chunk: q_i . dQ_i of what the accumulators hold now; this wave's
                 // half of the columns goes to LDS, the halves meet behind the next barrier
-                const T* Qh = reinterpret_cast<const T*>(a.Qrow) + offA + (size_t)dh * (D / 2);
+                // The wave's half row is 2 NP pieces of 8 columns; a lane holds four columns of every piece (8 bytes), which as
+                // loads of their own were 8 bytes of 32 rows per instruction: the lane half h loads the pieces NP h .. NP h + NP-1
+                // whole instead, and one swap per register pair hands each lane its four columns of every piece.  One row block
+                // at a time: with both blocks' pieces in flight the kernel spills at D = 256.  (Touching the rows' lines ahead
+                // of the state phase, as an L2 prefetch, cost more than it saved: measured.)
+                typedef int i32x4 __attribute__((ext_vector_type(4)));
+                typedef int i32x2 __attribute__((ext_vector_type(2)));
+                constexpr int HRB = (D / 2) * (int)sizeof(T), NP = row8_pieces_per_lane(HRB);
+                static_assert(NP == 2 * NDH, "a lane's pieces cover two of its column blocks' groups each");
+                const char* Qh = reinterpret_cast<const char*>(reinterpret_cast<const T*>(a.Qrow) + offA + (size_t)dh * (D / 2));
 #pragma unroll
                 for (int r = 0; r < 2; r++) {
                     float rp = 0.f;
+                    i32x4 wq[NP];
 #pragma unroll
-                    for (int d = 0; d < NDH; d++)
+                    for (int i = 0; i < NP; i++)
+                        wq[i] = *reinterpret_cast<const i32x4*>(Qh + (size_t)rowc[r] * rsA * sizeof(T) + row8_piece_offset(i, h, HRB));
 #pragma unroll
-                        for (int a4 = 0; a4 < 4; a4++) {
-                            const f32x4 qv = __builtin_convertvector(
-                                *reinterpret_cast<const typename R::vec4*>(Qh + (size_t)rowc[r] * rsA + 32 * d + 8 * a4 + 4 * h), f32x4);
+                    for (int i = 0; i < NP; i++) {
+                        // (lanes 32..63 of the first operand change places with lanes 0..31 of the second: result u is piece NP u + i)
+                        const auto s0 = __builtin_amdgcn_permlane32_swap(wq[i][0], wq[i][2], false, false);
+                        const auto s1 = __builtin_amdgcn_permlane32_swap(wq[i][1], wq[i][3], false, false);
+#pragma unroll
+                        for (int u = 0; u < 2; u++) {
+                            const f32x4 qv = __builtin_convertvector(__builtin_bit_cast(typename R::vec4, i32x2{(int)s0[u], (int)s1[u]}), f32x4);
+                            const int pc = NP * u + i, d = pc / 4, a4 = pc % 4;   // column block and group of four registers
 #pragma unroll
                             for (int c = 0; c < 4; c++) rp += oacc[r][d][4 * a4 + c] * qv[c];
                         }
+                    }
                     rp = sum_halves(rp);
                     if (h == 0) rix[((rg * 2 + dh) * 2 + r) * 32 + c32] = rp;
                 }
