@@ -32,7 +32,8 @@ struct Row8Cfg {
     static constexpr size_t PBUF_BYTES = 2 * 2 * 4 * 64 * 16;                          // [row group][row block][16-key group][lane] x 16 B
     // partial row sums [rg][kh][r][32] (forward) or the rows' 1/n and db [rg][r][32][2] (dQ pass), then the counters
     // (and [rg][half][r][32] floats for the row sums of the state part of a chunked dQ pass)
-    static constexpr size_t MISC_BYTES = 2 * 2 * 2 * 32 * sizeof(float) + 64 + 2 * 2 * 2 * 32 * sizeof(float);
+    // and the vector state n~ of the previous chunk (D floats)
+    static constexpr size_t MISC_BYTES = 2 * 2 * 2 * 32 * sizeof(float) + 64 + 2 * 2 * 2 * 32 * sizeof(float) + D * sizeof(float);
     static constexpr size_t FIXED_BYTES = 4 * TILE_BYTES + 2 * AUX_BYTES + PBUF_BYTES + MISC_BYTES;  // + NG doubles
 };
 
@@ -54,6 +55,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
     float* const bex = reinterpret_cast<float*>(smem + 4 * Cfg::TILE_BYTES + 2 * Cfg::AUX_BYTES + Cfg::PBUF_BYTES);
     unsigned* const pcnt = reinterpret_cast<unsigned*>(bex + 2 * 2 * 2 * 32);   // [2] fragments-copied counters
     float* const rix = bex + 2 * 2 * 2 * 32 + 16;
+    float* const nvl = rix + 2 * 2 * 2 * 32;   // [D]
     double* const sG = reinterpret_cast<double*>(smem + Cfg::FIXED_BYTES);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, h = lane >> 5, c32 = lane & 31;
@@ -134,8 +136,13 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
     // Every trip to memory in this prologue costs thousands of cycles, so the independent ones are requested back to back
     // and their values used as late as possible: the granule bases are asked for here and stored to LDS just before the
     // first barrier.
+    // (likewise the vector state of the previous chunk, D floats: fetched by the first D threads, read from LDS behind the
+    // state tiles and behind the tile loop -- as loads of their own there, each was one more trip to memory in the
+    // workgroup's chain of them, and a trip is 2 to 2.5 us with one workgroup per CU)
     const double g_mine = tid < NG ? a.G2[goff + tid] : 0.0;
+    const float n_mine = (chunk > 0 && tid < D) ? a.Nst[((size_t)bh * a.n_states + chunk - 1) * D + tid] : 0.f;
     auto store_granule_bases = [&]() {
+        if (chunk > 0 && tid < D) nvl[tid] = n_mine;
         if (tid < NG) sG[tid] = g_mine;
         for (int g = tid + 512; g < NG; g += 512) sG[g] = a.G2[goff + g];
     };
@@ -164,6 +171,12 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             for (int s = 0; s < NS; s++) xf[r][s] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, s, h);
             crow_base[r] = -0.5f * __log2f((float)D) - a.beta2[poff + rowc[r]];
         }
+        float dec_rows[2] = {0.f, 0.f};   // forward in chunks: the rows' decay since the end of the previous chunk (for the row sums)
+        if (MODE == R8_FWD && chunk > 0) {
+#pragma unroll
+            for (int r = 0; r < 2; r++)
+                dec_rows[r] = fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
+        }
         if constexpr (MODE == R8_DQ) {
             // Per-row scalars of the backward (1/n, db: see row_stats) for row block kh of the row group.  Behind the first
             // chunk the consumers start with the state tiles and this role would wait for them: it has the rows' dh
@@ -186,7 +199,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         for (int r = 0; r < 2; r++) {
 #pragma unroll
             for (int s = 0; s < NS; s++) pin(xf[r][s]);
-            pin(crow_base[r]); pin(inv_n[r]); pin(dbv[r]);
+            pin(crow_base[r]); pin(inv_n[r]); pin(dbv[r]); pin(dec_rows[r]);
         }
         SwzRowReaderX<T, D> krd;
         krd.init(lane);
@@ -394,10 +407,10 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         if constexpr (MODE == R8_FWD) {
             if (chunk > 0) {
                 // Row sums: what lies before the chunk contributes decay_i (q_i . n~) with the vector state n~ of the
-                // previous chunk; the two producers of a row group take half of the contraction each.  Done here, behind
-                // the tile loop, where this role has time to spare (the consumers are one tile behind): in the prologue
-                // the loads of n~ were one more trip to memory on the workgroup's critical path.
-                const float* nst = a.Nst + ((size_t)bh * a.n_states + chunk - 1) * D + 8 * h;
+                // previous chunk (in LDS since the prologue); the two producers of a row group take half of the contraction
+                // each.  Done here, behind the tile loop, where this role has time to spare (the consumers are one tile
+                // behind).
+                const float* nst = nvl + 8 * h;
                 float part[2] = {0.f, 0.f};
                 auto half_dot = [&](auto first_tag) {   // (the fragment index must be a constant: xf lives in registers)
                     constexpr int S0 = decltype(first_tag)::value;
@@ -415,8 +428,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (kh == 0) half_dot(std::integral_constant<int, 0>{});
                 else half_dot(std::integral_constant<int, NS / 2>{});
 #pragma unroll
-                for (int r = 0; r < 2; r++)
-                    bsum[r] += part[r] * fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
+                for (int r = 0; r < 2; r++) bsum[r] += part[r] * dec_rows[r];
             }
         }
         dma_wait();
@@ -543,6 +555,20 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
             }
         }
+        // (chunks: the rows' own X fragments for the first pair of state tiles are requested here, with everything else of
+        // the prologue, not behind the barrier: one trip to memory less in the workgroup's chain)
+        const T* const Xc = reinterpret_cast<const T*>(a.X) + offX;
+        frag pf0[2][4], pf1[2][4];
+        auto load_pf = [&](int pp) {
+#pragma unroll
+            for (int r = 0; r < 2; r++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    pf0[r][g] = frag_rowmajor<T>(Xc + (size_t)rowc[r] * rsX, 4 * pp + g, h);
+                    pf1[r][g] = frag_rowmajor<T>(Xc + (size_t)rowc[r] * rsX, 4 * pp + 4 + g, h);
+                }
+        };
+        if (chunk > 0) load_pf(0);
         store_granule_bases();
         __syncthreads();
         if (chunk > 0) {
@@ -552,29 +578,21 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
             // from global memory: the state's rows are stored in the order in which this product contracts them.
             //   forward: H^T += C~^T-tiles x Q^T, then the rows' decay exp(A_e - A_i)
             //   dQ pass: dQ^T += C~-tiles x dH^T, then decay / n; and the rank-one term decay * db_i * n~
-            const T* X = reinterpret_cast<const T*>(a.X) + offX;
             auto none = [](int, int) {};
 #pragma unroll 1
             for (int pp = 0; pp < D / 64; pp += 2) {
                 if (pp > 0) {
                     tdma.issue(sa, Cst + (size_t)GRAN * pp * D);
                     tdma.issue(sb, Cst + (size_t)GRAN * (pp + 1) * D);
+                    load_pf(pp);
                 }
-                frag pf0[2][4], pf1[2][4];
-#pragma unroll
-                for (int r = 0; r < 2; r++)
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        pf0[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, 4 * pp + g, h);
-                        pf1[r][g] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, 4 * pp + 4 + g, h);
-                    }
                 dma_wait();
                 __syncthreads();
                 gemm2(sa, pf0, none);
                 gemm2(sb, pf1, none);
                 __syncthreads();   // both stages are free again
             }
-            const float* nst = a.Nst + ((size_t)bh * a.n_states + chunk - 1) * D + (size_t)dh * (D / 2) + 4 * h;
+            const float* nst = nvl + dh * (D / 2) + 4 * h;
 #pragma unroll
             for (int r = 0; r < 2; r++) {
                 float dec = dec_pre[r];
