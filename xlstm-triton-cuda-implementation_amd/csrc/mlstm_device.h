@@ -559,6 +559,15 @@ template <typename T> __device__ __forceinline__ float to_f32(T x) { return (flo
 // sum_j C~_ij (dh_i . v_j) = n_i (dh_i . h_i) it collapses to one dot product per row.
 // hrow_lo (may be null): the remainder h - (h rounded to the element type), left by a forward in split mode; with it
 // the dot product sees h to about 16 significant bits.
+// 1/n and db of a row from delta = dh . h, the normaliser sum b and the stabiliser m (mlstm_matmul.py:194-196)
+__device__ __forceinline__ void row_stats_of(float delta, float b, float m, float& inv_n, float& db) {
+    const float em = __expf(-m);
+    inv_n = 1.0f / (fmaxf(fabsf(b), em) + 1e-6f);
+    const float dn = -delta * inv_n;
+    const float sg = (b > 0.f) ? 1.f : ((b < 0.f) ? -1.f : 0.f);
+    db = (fabsf(b) > em) ? sg * dn : 0.f;
+}
+
 template <typename T, int NS>
 __device__ __forceinline__ void row_stats(const typename Tr<T>::frag (&xf)[NS], const T* hrow, int h, float b, float m, float& inv_n,
                                           float& db, const T* hrow_lo = nullptr) {
@@ -579,12 +588,7 @@ __device__ __forceinline__ void row_stats(const typename Tr<T>::frag (&xf)[NS], 
         }
         acc += acc_lo;
     }
-    const float delta = sum_halves(acc);
-    const float em = __expf(-m);
-    inv_n = 1.0f / (fmaxf(fabsf(b), em) + 1e-6f);
-    const float dn = -delta * inv_n;
-    const float sg = (b > 0.f) ? 1.f : ((b < 0.f) ? -1.f : 0.f);
-    db = (fabsf(b) > em) ? sg * dn : 0.f;
+    row_stats_of(sum_halves(acc), b, m, inv_n, db);
 }
 
 __device__ __forceinline__ float log_sigmoid(float x) {

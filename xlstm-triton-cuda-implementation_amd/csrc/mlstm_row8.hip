@@ -153,12 +153,32 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
     const auto ra = tdma.rows(rtid, (unsigned)(rsA * sizeof(T)));   // Y1, Y2 tiles
     constexpr int PW = TileDma<T, D, GRAN, 256>::PER_WAVE;
     frag* const p_rg = pbuf + rg * (2 * 4 * 64) + lane;        // fragment (r, g) of the row group -> p_rg[(4*r + g) * 64]
+    // The workgroup's 128 rows of X (Q in the forward, dH in the dQ pass) are operands of every product here, a fragment per
+    // lane and contraction step.  Straight from memory that is 16 bytes of a row per lane, 32 rows per instruction, by four
+    // waves per row group for the same rows (knocked out, those loads were 16 us of the forward's 113 and 11 of the dQ pass's
+    // 133 at B4 H8 S4096 D256).  The rows come in once instead, as two 64-row tiles in whole lines -- row group 0 by the
+    // producers into a Y1 stage, row group 1 by the consumers into a Y2 stage -- and every wave reads its fragments from
+    // there behind the first barrier.  Behind the first chunk the FIRST stages serve (the second ones hold state tiles), and
+    // the first key tiles follow into them once the first pair of state tiles is done with; in the first chunk, and without
+    // chunks, the SECOND stages serve, which the tiles' copies reach only behind a later barrier.
+    const int xst = chunk > 0 ? 0 : 1;
+    const T* const xtile = reinterpret_cast<const T*>((rg ? y2s : y1s) + xst * Cfg::TILE_BYTES);   // the wave's row group's rows
+    auto x_copy = [&]() {   // (this role's tile: producers row group 0, consumers row group 1)
+        const T* Xg = reinterpret_cast<const T*>(a.X) + (MODE == R8_FWD ? offA : offB);
+        const size_t rs = MODE == R8_FWD ? rsA : rsB;
+        const int row0 = q0 + (producer ? 0 : GRAN);
+        T* dst = reinterpret_cast<T*>((producer ? y1s : y2s) + xst * Cfg::TILE_BYTES);
+        if (row0 + GRAN <= S) tdma.issue(dst, Xg + (size_t)row0 * rs, tdma.rows(rtid, (unsigned)(rs * sizeof(T))));
+        else tile_dma<T, D, GRAN, 256>(dst, Xg, row0 < S ? row0 : S - 1, S, rtid, rs);
+    };
+    SwzRowReaderX<T, D> xrd;
+    xrd.init(lane);
 
     if (producer) {
         // ------------------------------------------------------------------------------------------ producers
         const int kh = sub;
-        const T* X = reinterpret_cast<const T*>(a.X) + offX;
-        {   // first of all the copy of the first Y1 tile: its latency then overlaps that of the plain loads below
+        x_copy();
+        if (chunk == 0) {   // the copy of the first Y1 tile (behind the first chunk it follows the first pair of state tiles)
             T* dst = reinterpret_cast<T*>(y1s);
             if (0 < full_tiles) tdma.issue(dst, Y1, ra);
             else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
@@ -166,41 +186,30 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         frag xf[2][NS];
         float crow_base[2], inv_n[2] = {0.f, 0.f}, dbv[2] = {0.f, 0.f}, bsum[2] = {0.f, 0.f};
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-#pragma unroll
-            for (int s = 0; s < NS; s++) xf[r][s] = frag_rowmajor<T>(X + (size_t)rowc[r] * rsX, s, h);
-            crow_base[r] = -0.5f * __log2f((float)D) - a.beta2[poff + rowc[r]];
-        }
+        for (int r = 0; r < 2; r++) crow_base[r] = -0.5f * __log2f((float)D) - a.beta2[poff + rowc[r]];
         float dec_rows[2] = {0.f, 0.f};   // forward in chunks: the rows' decay since the end of the previous chunk (for the row sums)
         if (MODE == R8_FWD && chunk > 0) {
 #pragma unroll
             for (int r = 0; r < 2; r++)
                 dec_rows[r] = fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
         }
-        if constexpr (MODE == R8_DQ) {
-            // Per-row scalars of the backward (1/n, db: see row_stats) for row block kh of the row group.  Behind the first
-            // chunk the consumers start with the state tiles and this role would wait for them: it has the rows' dh
-            // fragments in registers already and does the dot products with h itself.  (In the first chunk, and without
-            // chunks, it is the other way round: this role heads the critical path and the consumers idle.)
-            if (chunk > 0) {
-                float inv = 0.f, dbr = 0.f;
-                const int rc = rowc[kh];
-                const T* hrow = reinterpret_cast<const T*>(a.Hin) + offH + (size_t)rc * rsH;
-                if (kh == 0) row_stats<T, NS>(xf[0], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
-                else row_stats<T, NS>(xf[1], hrow, h, a.Bin[hoff + rc], a.M[hoff + rc], inv, dbr);
-                const int row = r0 + 32 * kh + c32;
-                if (h == 0) {
-                    *reinterpret_cast<float2*>(bex + ((rg * 2 + kh) * 32 + c32) * 2) = make_float2(inv, dbr);
-                    if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
-                }
-            }
+        // dQ pass behind the first chunk: this role forms the per-row scalars of the backward (1/n, db: see row_stats) for row
+        // block kh of the row group, while the consumers work through the state tiles (which need them only at the end).  The
+        // rows of h are requested here; the dot products with dh follow behind the barrier, when the dh fragments are there.
+        // (In the first chunk, and without chunks, it is the other way round: this role heads the critical path and the
+        // consumers, idle until the first P, form the scalars.)
+        frag hfr[NS];
+        float b_row = 0.f, m_row = 0.f;
+        if (MODE == R8_DQ && chunk > 0) {
+            const int rc = rowc[kh];
+            const T* hrow = reinterpret_cast<const T*>(a.Hin) + offH + (size_t)rc * rsH;
+#pragma unroll
+            for (int s = 0; s < NS; s++) hfr[s] = frag_rowmajor<T>(hrow, s, h);
+            b_row = a.Bin[hoff + rc];
+            m_row = a.M[hoff + rc];
         }
 #pragma unroll
-        for (int r = 0; r < 2; r++) {
-#pragma unroll
-            for (int s = 0; s < NS; s++) pin(xf[r][s]);
-            pin(crow_base[r]); pin(inv_n[r]); pin(dbv[r]); pin(dec_rows[r]);
-        }
+        for (int r = 0; r < 2; r++) { pin(crow_base[r]); pin(dec_rows[r]); }
         SwzRowReaderX<T, D> krd;
         krd.init(lane);
         const float* const alpha_head = a.alpha2 + poff;
@@ -340,17 +349,50 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         };
 
         store_granule_bases();
-        __syncthreads();  // sG, counters visible; plain global loads above are done (pin)
-        if constexpr (MODE == R8_DQ) {   // 1/n and db of the wave's rows, computed by the consumers while this role loaded its rows
+        dma_wait();
+        __syncthreads();  // sG, counters visible; the X tiles have landed
+        if (MODE == R8_DQ && chunk > 0) {   // (before the wave takes all its X fragments: the rows of h leave their registers first)
+            float acc = 0.f;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const frag xk = xrd.read(xtile, kh, s);
+#pragma unroll
+                for (int e = 0; e < R::EPL; e++) acc += (float)xk[e] * (float)hfr[s][e];
+            }
+            float inv = 0.f, dbr = 0.f;
+            row_stats_of(sum_halves(acc), b_row, m_row, inv, dbr);
+            const int row = r0 + 32 * kh + c32;
+            if (h == 0) {
+                *reinterpret_cast<float2*>(bex + ((rg * 2 + kh) * 32 + c32) * 2) = make_float2(inv, dbr);
+                if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int s = 0; s < NS; s++) xf[r][s] = xrd.read(xtile, r, s);
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int s = 0; s < NS; s++) pin(xf[r][s]);
+        if (chunk > 0) {   // the consumers work through the state tiles: two barriers per pair of tiles
+#pragma unroll
+            for (int pp = 0; pp < D / 64; pp += 2) {
+                __syncthreads();
+                __syncthreads();
+                if (pp == 0) {   // every wave is done with the X tiles: the first Y1 tile follows into its stage
+                    T* dst = reinterpret_cast<T*>(y1s);
+                    if (0 < full_tiles) tdma.issue(dst, Y1, ra);
+                    else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
+                }
+            }
+        }
+        if constexpr (MODE == R8_DQ) {   // 1/n and db of the wave's rows (written ahead of the last barrier passed, by either role)
 #pragma unroll
             for (int r = 0; r < 2; r++) {
                 const float2 st = *reinterpret_cast<const float2*>(bex + ((rg * 2 + r) * 32 + c32) * 2);
                 inv_n[r] = st.x; dbv[r] = st.y;
             }
-        }
-        if (chunk > 0) {   // the consumers work through the state tiles: two barriers per pair of tiles
-#pragma unroll
-            for (int pp = 0; pp < D / 64; pp += 2) { __syncthreads(); __syncthreads(); }
         }
         const double GI = sG[(wave_active ? r0 : S - 1) / GRAN];
         aux_dma(0);
@@ -530,6 +572,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         }
         // per-row scalars that are only needed late (the rows' decay since the end of the previous chunk; the forward's
         // stabiliser for the normaliser): requested now, so that their trip to memory is not waited for then
+        x_copy();
         float dec_pre[2] = {1.f, 1.f}, m_pre[2] = {0.f, 0.f};
 #pragma unroll
         for (int r = 0; r < 2; r++) {
@@ -537,7 +580,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 dec_pre[r] = fast_exp2(a.beta2[poff - 1] - a.beta2[poff + rowc[r]] + (float)(a.G2[goff + rowc[r] / GRAN] - a.G2[goff - 1]));
             if constexpr (MODE == R8_FWD) m_pre[r] = a.M[hoff + rowc[r]];
         }
-        y2_bulk(0);
+        if (chunk == 0) y2_bulk(0);   // (behind the first chunk the first Y2 tile follows the first pair of state tiles)
         if (MODE == R8_DQ && chunk == 0) {
             // Per-row scalars of the backward for row block r = dh of the row group (the producers need them from their
             // first tile on, the column kernel reads them from global memory): this role idles until the first P arrives.
@@ -555,11 +598,9 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (row < S) { a.inv_n[poff + row] = inv; a.db[poff + row] = dbr; }
             }
         }
-        // (chunks: the rows' own X fragments for the first pair of state tiles are requested here, with everything else of
-        // the prologue, not behind the barrier: one trip to memory less in the workgroup's chain)
         const T* const Xc = reinterpret_cast<const T*>(a.X) + offX;
         frag pf0[2][4], pf1[2][4];
-        auto load_pf = [&](int pp) {
+        auto load_pf = [&](int pp) {   // the rows' X fragments for the pair of state tiles pp, pp + 1, from memory
 #pragma unroll
             for (int r = 0; r < 2; r++)
 #pragma unroll
@@ -568,9 +609,15 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                     pf1[r][g] = frag_rowmajor<T>(Xc + (size_t)rowc[r] * rsX, 4 * pp + 4 + g, h);
                 }
         };
-        if (chunk > 0) load_pf(0);
         store_granule_bases();
-        __syncthreads();
+        dma_wait();
+        __syncthreads();   // sG, counters visible; the X tiles (and behind the first chunk the first state tiles) have landed
+        if (chunk > 0) {   // (the first pair's fragments out of the X tile)
+#pragma unroll
+            for (int r = 0; r < 2; r++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) { pf0[r][g] = xrd.read(xtile, r, g); pf1[r][g] = xrd.read(xtile, r, 4 + g); }
+        }
         if (chunk > 0) {
             // What lies before the chunk: the state at the end of the previous chunk, D rows of D entries, as D/64 tiles
             // through the second stages of Y1 and Y2 (free until the first key tile has been worked on), two at a time.
@@ -591,6 +638,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 gemm2(sa, pf0, none);
                 gemm2(sb, pf1, none);
                 __syncthreads();   // both stages are free again
+                if (pp == 0) y2_bulk(0);   // (and so are the X tiles' stages: the first Y2 tile follows into its own)
             }
             const float* nst = nvl + dh * (D / 2) + 4 * h;
 #pragma unroll
