@@ -631,12 +631,22 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (pp > 0) {
                     tdma.issue(sa, Cst + (size_t)GRAN * pp * D);
                     tdma.issue(sb, Cst + (size_t)GRAN * (pp + 1) * D);
-                    load_pf(pp);
+                    if (pp > 2) load_pf(pp);   // (the second pair's fragments came out of the X tile: below)
                 }
                 dma_wait();
                 __syncthreads();
                 gemm2(sa, pf0, none);
                 gemm2(sb, pf1, none);
+                if (pp == 0 && D / 64 > 2) {   // the next pair's fragments, while the X tile is still there
+#pragma unroll
+                    for (int r = 0; r < 2; r++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++) { pf0[r][g] = xrd.read(xtile, r, 8 + g); pf1[r][g] = xrd.read(xtile, r, 12 + g); }
+#pragma unroll
+                    for (int r = 0; r < 2; r++)
+#pragma unroll
+                        for (int g = 0; g < 4; g++) { pin(pf0[r][g]); pin(pf1[r][g]); }
+                }
                 __syncthreads();   // both stages are free again
                 if (pp == 0) y2_bulk(0);   // (and so are the X tiles' stages: the first Y2 tile follows into its own)
             }
