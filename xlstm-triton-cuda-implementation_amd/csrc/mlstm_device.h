@@ -263,6 +263,27 @@ __device__ __forceinline__ void tile_dma(T* tile, const T* g, int row0, int S, i
     }
 }
 
+// The same copy as a loop that stays a loop, for the places where it rarely runs (a sequence's last, partial tile) but would
+// otherwise keep one 64-bit address per block alive across code that needs every register.
+template <typename T, int D, int ROWS, int NT>
+__device__ __forceinline__ void tile_dma_rolled(T* tile, const T* g, int row0, int S, int tid, size_t row_stride = D) {
+    using Z = Swz<T, D>;
+    constexpr int NW = NT / 64, BLOCKS = ROWS * Z::CPR / 64;
+    static_assert(BLOCKS % NW == 0, "tile must divide evenly over the waves");
+    const int wave = tid >> 6, lane = tid & 63;
+    const unsigned base = lds_offset_of(tile);
+#pragma unroll 1
+    for (int it = 0; it < BLOCKS / NW; it++) {
+        const int blk = it * NW + wave;
+        const int p = blk * 64 + lane;
+        const int r = p / Z::CPR, pc = p % Z::CPR;
+        const int c = pc ^ Z::key(r);
+        int gr = row0 + r;
+        gr = gr < S ? gr : S - 1;
+        dma16(g + (size_t)gr * row_stride + c * Z::EPC, __builtin_amdgcn_readfirstlane(base + blk * 1024));
+    }
+}
+
 // Same copy with everything that does not change from tile to tile hoisted out of the loop: the per-lane byte offsets
 // inside a tile are computed once (init), a tile is addressed by a scalar base pointer, and the LDS destinations are
 // scalar arithmetic on the wave index.  A tile then costs no vector ALU work at all: per 1 KB block one s_mov to M0

@@ -168,8 +168,9 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         const size_t rs = MODE == R8_FWD ? rsA : rsB;
         const int row0 = q0 + (producer ? 0 : GRAN);
         T* dst = reinterpret_cast<T*>((producer ? y1s : y2s) + xst * Cfg::TILE_BYTES);
-        if (row0 + GRAN <= S) tdma.issue(dst, Xg + (size_t)row0 * rs, tdma.rows(rtid, (unsigned)(rs * sizeof(T))));
-        else tile_dma<T, D, GRAN, 256>(dst, Xg, row0 < S ? row0 : S - 1, S, rtid, rs);
+        // (the per-lane row offsets of the Y tiles serve when X has their stride)
+        if (row0 + GRAN <= S) tdma.issue(dst, Xg + (size_t)row0 * rs, (MODE == R8_FWD || DENSE) ? ra : tdma.rows(rtid, (unsigned)(rs * sizeof(T))));
+        else tile_dma_rolled<T, D, GRAN, 256>(dst, Xg, row0 < S ? row0 : S - 1, S, rtid, rs);
     };
     SwzRowReaderX<T, D> xrd;
     xrd.init(lane);
@@ -181,7 +182,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         if (chunk == 0) {   // the copy of the first Y1 tile (behind the first chunk it follows the first pair of state tiles)
             T* dst = reinterpret_cast<T*>(y1s);
             if (0 < full_tiles) tdma.issue(dst, Y1, ra);
-            else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
+            else tile_dma_rolled<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
         }
         frag xf[2][NS];
         float crow_base[2], inv_n[2] = {0.f, 0.f}, dbv[2] = {0.f, 0.f}, bsum[2] = {0.f, 0.f};
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         auto y1_bulk = [&](int j) {
             T* dst = reinterpret_cast<T*>(y1s + (j & 1) * Cfg::TILE_BYTES);
             if (j < full_tiles) tdma.issue(dst, Y1 + (size_t)GRAN * j * rsA, ra);
-            else tile_dma<T, D, GRAN, 256>(dst, Y1, GRAN * j, S, rtid, rsA);
+            else tile_dma_rolled<T, D, GRAN, 256>(dst, Y1, GRAN * j, S, rtid, rsA);
             aux_dma(j);
         };
         // s_r = (32 keys of this wave) x (row block r); every Y1 fragment feeds both row blocks.  The operand reads run
@@ -383,7 +384,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
                 if (pp == 0) {   // every wave is done with the X tiles: the first Y1 tile follows into its stage
                     T* dst = reinterpret_cast<T*>(y1s);
                     if (0 < full_tiles) tdma.issue(dst, Y1, ra);
-                    else tile_dma<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
+                    else tile_dma_rolled<T, D, GRAN, 256>(dst, Y1, 0, S, rtid, rsA);
                 }
             }
         }
@@ -531,7 +532,7 @@ __global__ __launch_bounds__(512) void row8_kernel(RowArgs a) {
         auto y2_bulk = [&](int j) {
             T* dst = reinterpret_cast<T*>(y2s + (j & 1) * Cfg::TILE_BYTES);
             if (j < full_tiles) tdma.issue(dst, Y2 + (size_t)GRAN * j * rsA, ra);
-            else tile_dma<T, D, GRAN, 256>(dst, Y2, GRAN * j, S, rtid, rsA);
+            else tile_dma_rolled<T, D, GRAN, 256>(dst, Y2, GRAN * j, S, rtid, rsA);
         };
         // fragments of one tile into registers, then tell the producers their buffer is free again
         auto take = [&](frag (&pf)[2][4]) {
