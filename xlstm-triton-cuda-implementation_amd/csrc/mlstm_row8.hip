@@ -14,6 +14,8 @@
 // buffer of a row group is handed back from its two consumers to its two producers through an LDS counter: a
 // consumer copies its fragments into registers first thing after the barrier and bumps the counter; the producers
 // check it only when they are about to publish the next tile's P, long after.
+// The rows' own operand (Q in the forward, dH in the dQ pass) comes in once per workgroup, as two 64-row tiles through
+// stages that are idle at that point, and every wave takes its fragments from there (see x_copy).
 // MODE_FWD replaces mlstm_matmul_kernel (mlstm_matmul.py:38-101) and the CUDA kernel mlstm_forward
 // (cuda-src/mlstm_forward.cu:14-189); MODE_DQ the dQ loop of mlstm_matmul_kernel_backward (mlstm_matmul.py:239-267).
 #include <type_traits>
